@@ -1,0 +1,172 @@
+/* mlora.h -- C ABI of the MI355X (gfx950) multi-LoRA batching operator.
+ *
+ * Plain pointers and sizes only; every pointer marked "device" is device memory owned by the
+ * caller, every launch goes on the caller's stream, the library allocates nothing and keeps no
+ * state between calls.  Every function returns MLORA_OK (0) or a negative mlora_status;
+ * mlora_last_error() then returns a message for the calling thread.
+ *
+ * Citations name the reference interface each entry point replaces (paths relative to the
+ * mi150/VaLoRA checkout).
+ */
+#ifndef MLORA_H_
+#define MLORA_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { MLORA_F16 = 0, MLORA_BF16 = 1 } mlora_dtype;
+
+typedef enum {
+  MLORA_OK = 0,
+  MLORA_ERR_INVALID = -1,     /* bad argument (null pointer, negative size, misaligned base) */
+  MLORA_ERR_NO_KERNEL = -2,   /* "No suitable kernel." -- valora/csrc/lora_ops.cc:124-125 */
+  MLORA_ERR_WORKSPACE = -3,   /* workspace or plan buffer too small */
+  MLORA_ERR_LAUNCH = -4       /* the HIP runtime refused a launch */
+} mlora_status;
+
+/* Behaviour switches of the shrink store (see mlora_shrink_finish). */
+enum {
+  MLORA_SHRINK_OVERWRITE = 0, /* y[t,:r] = v, columns >= r untouched (BGMV, bgmv_impl.cuh:36,147) */
+  MLORA_SHRINK_ZERO_PAD = 1,  /* y[t,:width] = v, zero for columns >= r (Triton, lora_prefill.py:89,96-100) */
+  MLORA_SHRINK_ACCUMULATE = 2 /* y[t,:r] += v (ATMM beta = 1, atmm/.../bgmv_impl.cuh:174) */
+};
+
+/* Pool + adapter index operands shared by all op entry points (device pointers).
+ * Semantics: valora/server/router/model_infer/infer_adapter.py:14-17,128-148.            */
+typedef struct {
+  const void *w;            /* pool rows, 16-bit elements, row stride = the call's wide dim     */
+  int64_t w_rows;           /* number of pool rows (rows named by a_loc outside it are skipped) */
+  const int64_t *a_start;   /* [n_adapters] offset into a_loc                                   */
+  const int64_t *a_len;     /* [n_adapters] n_slots * rank                                      */
+  const int64_t *a_loc;     /* [a_loc_len] pool row per (adapter, slot, rank row)               */
+  int64_t n_adapters;
+  int64_t a_loc_len;
+  int32_t n_slots;          /* 4 in the reference (q,k,v,o): bgmv_impl.cuh:35                   */
+} mlora_pool;
+
+/* Host-side handle of a plan: the device buffer (caller-owned, mlora_plan_bytes() bytes) plus
+ * the shape it was built for.  mlora_build_plan fills every field but dev and bytes.          */
+typedef struct {
+  void *dev;
+  size_t bytes;
+  int64_t T;
+  int64_t n_adapters;
+  int32_t bm_shrink;        /* tile heights in tokens the two tile lists were cut with          */
+  int32_t bm_expand;
+} mlora_plan;
+
+const char *mlora_last_error(void);
+int mlora_version(void);
+
+/* ---- sizing ------------------------------------------------------------------------------ */
+/* Bytes of a plan for T tokens and n_adapters adapters.                                       */
+size_t mlora_plan_bytes(int64_t T, int64_t n_adapters);
+/* Bytes of the fp32 split-K partial buffer the shrink writes and the expand reads.            */
+size_t mlora_partial_bytes(int64_t T, int64_t max_rank, int32_t ksplit);
+/* Bytes of scratch the one-call entry points (dispatch_bgmv, dispatch_sgmm, prefill_*) need.
+ * Replaces sgmm_tmp_size (atmm/valora/csrc/bgmv/bgmv_impl.cuh:128-132).                       */
+size_t mlora_workspace_bytes(int64_t T, int64_t n_adapters, int64_t max_rank);
+
+/* ---- index / segment builders ------------------------------------------------------------- */
+/* Adapter-grouped work tiles from per-token adapter ids (device int64[T]; an id outside
+ * [0, n_adapters) or an adapter of rank 0 marks a token that gets no LoRA).  Stable counting
+ * sort of the tokens by adapter + one tile list per tile height.  Replaces the host-side
+ * grouping done by precompute_sgmm_args_* (atmm/valora/csrc/bgmv/bgmv_impl.cuh:76-125).
+ * bm_shrink, bm_expand: tile heights in tokens (16, 32 or 64 / any multiple of 16 up to 256);
+ * 0 lets the library choose.                                                                 */
+int mlora_build_plan(void *stream, mlora_plan *plan, const int64_t *ids, int64_t T,
+                     const int64_t *a_start, const int64_t *a_len, int64_t n_adapters,
+                     int32_t n_slots, int32_t bm_shrink, int32_t bm_expand);
+
+/* Run-length encoding of per-token ids, bit-exact with count_consecutive_requests
+ * (atmm/valora/csrc/bgmv/bgmv_impl.cuh:39-72).  Outputs are device int64 arrays with room for
+ * T entries; only the first *num_runs entries are written.  num_runs: device int64[1].        */
+int mlora_count_consecutive(void *stream, const int64_t *lora_rank, int64_t n_adapters,
+                            const int64_t *indicies, int64_t T, int64_t *output_counts,
+                            int64_t *rank_counts, int64_t *lora_ids, int64_t *start_ids,
+                            int64_t *num_runs);
+
+/* ids_out[t] = ids_in[t] for rows covered by problems i < P (rows start_ids[i] ..
+ * start_ids[i] + output_counts[i]), -1 elsewhere.  Turns the ATMM segment tensors
+ * (atmm/valora/csrc/lora_ops.cc:115-122) into per-token ids.                                  */
+int mlora_ids_from_segments(void *stream, int64_t *ids_out, const int64_t *ids_in,
+                            const int64_t *start_ids, const int64_t *output_counts, int64_t P,
+                            int64_t T);
+
+/* ids_out[b_start_loc[i] + m] = b_indicies[i] for m < min(b_seq_len[i], max_rows), -1 elsewhere
+ * (per-request operands of valora/models/peft/triton_kernel/lora/lora_prefill.py:105,139).    */
+int mlora_ids_from_requests(void *stream, int64_t *ids_out, const int32_t *b_start_loc,
+                            const int32_t *b_seq_len, const int64_t *b_indicies, int64_t n_req,
+                            int64_t T, int64_t max_rows);
+
+/* ---- planned op: shrink / expand / fused ---------------------------------------------------- */
+/* partial[s][p][R] (fp32) = sum over K-chunk s of x[perm[p], k] * A[j, k]; p = sorted position.
+ * Kernel semantics: valora/csrc/bgmv/bgmv_impl.cuh:14-148.                                    */
+int mlora_shrink_partial(void *stream, const mlora_plan *plan, float *partial, size_t partial_bytes,
+                         const void *x, int64_t T, int64_t h_in, int64_t max_rank,
+                         const mlora_pool *pool, int32_t slot, int32_t ksplit, mlora_dtype dtype);
+
+/* y[perm[p], j] (<-|+=) T(sum_s partial[s][p][j]); mode is one of MLORA_SHRINK_*; y has row
+ * stride y_stride elements and `width` is the number of columns mode ZERO_PAD fills.          */
+int mlora_shrink_finish(void *stream, const mlora_plan *plan, const float *partial, void *y,
+                        int64_t T, int64_t y_stride, int64_t max_rank, int32_t ksplit,
+                        int32_t mode, int32_t width, mlora_dtype dtype);
+
+/* y[t,:] = T(y[t,:] + scale[a] * T(v[t,:r]) * B_a).  v comes either from `partial`
+ * (summed over ksplit, rounded to T once -- the reference holds it as a T tensor between its
+ * two launches) or, when partial == NULL, from xv (a T matrix [T, v_stride]).
+ * Kernel semantics: valora/csrc/bgmv/bgmv_impl.cuh:152-207.                                   */
+int mlora_expand(void *stream, const mlora_plan *plan, void *y, int64_t T, int64_t h_out,
+                 const float *partial, int32_t ksplit, const void *xv, int64_t v_stride,
+                 int64_t max_rank, const mlora_pool *pool, int32_t slot, const void *scales,
+                 mlora_dtype dtype);
+
+/* Shrink + expand of one target in one call (two launches, v stays in `partial`).  pool_a holds
+ * the A rows (row width h_in), pool_b the B rows (row width h_out); they share the index.     */
+int mlora_lora_apply(void *stream, const mlora_plan *plan, float *partial, size_t partial_bytes,
+                     void *y, const void *x, int64_t T, int64_t h_in, int64_t h_out,
+                     int64_t max_rank, const mlora_pool *pool_a, const mlora_pool *pool_b,
+                     int32_t slot, const void *scales, int32_t ksplit, mlora_dtype dtype);
+
+/* ---- the reference's entry points, one call each -------------------------------------------- */
+/* dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales)
+ * valora/csrc/lora_ops.cc:76-126.  Direction: h_in < h_out => expand, else shrink
+ * (valora/csrc/bgmv/bgmv_impl.cuh:221).                                                       */
+int mlora_dispatch_bgmv(void *stream, void *y, const void *x, const mlora_pool *pool,
+                        const int64_t *indicies, int64_t qkvo, const void *lora_scales, int64_t T,
+                        int64_t h_in, int64_t h_out, mlora_dtype dtype, void *workspace,
+                        size_t workspace_bytes);
+
+/* dispatch_bgmv of the ATMM extension (imported as dispatch_sgmm)
+ * atmm/valora/csrc/lora_ops.cc:115-186.  Rows of problems i < num_problems are processed with
+ * the adapter named by their per-token id; tile arguments tb_* / wp_* are accepted and ignored
+ * (tile selection is the library's own table).  shrink_mode: MLORA_SHRINK_OVERWRITE or
+ * MLORA_SHRINK_ACCUMULATE.                                                                     */
+int mlora_dispatch_sgmm(void *stream, void *y, const void *x, const mlora_pool *pool,
+                        const int64_t *indicies, int64_t qkvo, const void *lora_scales,
+                        const int64_t *output_counts, const int64_t *start_ids,
+                        int64_t num_problems, int64_t T, int64_t h_in, int64_t h_out,
+                        mlora_dtype dtype, int32_t shrink_mode, void *workspace,
+                        size_t workspace_bytes);
+
+/* lora_get_qkvo_fwd_shrink / lora_get_qkvo_fwd_expand
+ * valora/models/peft/triton_kernel/lora/lora_prefill.py:139-163 / :105-135.                   */
+int mlora_prefill_shrink(void *stream, void *o, const void *x, const mlora_pool *pool,
+                         const int32_t *b_start_loc, const int32_t *b_seq_len,
+                         const int64_t *b_indicies, int64_t n_req, int64_t T, int64_t hidden,
+                         int64_t o_stride, int64_t qkvo, int64_t max_rank, int64_t max_input_len,
+                         mlora_dtype dtype, void *workspace, size_t workspace_bytes);
+int mlora_prefill_expand(void *stream, void *o, const void *x, const mlora_pool *pool,
+                         const void *scale, const int32_t *b_start_loc, const int32_t *b_seq_len,
+                         const int64_t *b_indicies, int64_t n_req, int64_t T, int64_t x_stride,
+                         int64_t feat_out, int64_t qkvo, int64_t max_rank, int64_t max_input_len,
+                         mlora_dtype dtype, void *workspace, size_t workspace_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLORA_H_ */

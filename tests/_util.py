@@ -1,0 +1,79 @@
+"""Helpers shared by the parity tests: run one target of a workload through each entry point of
+the product (always through the C ABI) and through the CPU oracle."""
+import torch
+
+from oracle import lora_oracle as O
+
+MAX_ABS = 2e-2   # tolerance stated by the benchmark definition: max-abs error
+REL_L2 = 1e-3    # and relative L2 error, both against the reference semantics with fp32 accumulation
+
+
+def oracle_target(w, name, round_v=True):
+    t = w.target(name)
+    p = t.pool
+    return O.lora_op(w.y0[name], w.x[t.h_in], p_kb(w, name), p.value_buffer, p.a_start, p.a_len, p.a_loc,
+                     w.ids, t.slot, p.a_scaling, round_v=round_v)
+
+
+def p_kb(w, name):
+    return w.target(name).pool.key_buffer
+
+
+def max_rank(w):
+    return max(w.targets[0].pool.ranks)
+
+
+def run_bgmv(wd, name):
+    """Two dispatch_bgmv calls with a T-typed delta between them, like the reference caller
+    (valora/models/peft/lora_unordered_batch_infer.py:632-638)."""
+    from valora_amd.kernels import dispatch_bgmv
+    t = wd.target(name); p = t.pool
+    y = wd.y0[name].clone()
+    delta = torch.zeros(wd.T, max_rank(wd), dtype=wd.dtype, device=y.device)
+    dispatch_bgmv(delta, wd.x[t.h_in], p.key_buffer, p.a_start, p.a_len, p.a_loc, wd.ids, t.slot, p.a_scaling)
+    dispatch_bgmv(y, delta, p.value_buffer, p.a_start, p.a_len, p.a_loc, wd.ids, t.slot, p.a_scaling)
+    return y, delta
+
+
+def run_plan(wd, name, **kw):
+    from valora_amd.plan import LoraPlan
+    t = wd.target(name); p = t.pool
+    plan = LoraPlan(wd.ids, p.a_start, p.a_len, max_rank(wd), hidden=t.h_in, **kw)
+    y = wd.y0[name].clone()
+    plan.apply(y, wd.x[t.h_in], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
+    return y
+
+
+def run_sgmm(wd, name):
+    from valora_amd.atmm_ops import dispatch_bgmv as dispatch_sgmm
+    from valora_amd.segments import count_consecutive_requests
+    t = wd.target(name); p = t.pool
+    oc, rc, li, st, num = count_consecutive_requests(p.a_len, wd.ids)
+    P = int(num.item())
+    y = wd.y0[name].clone()
+    delta = torch.zeros(wd.T, max_rank(wd), dtype=wd.dtype, device=y.device)
+    tmp = torch.zeros(max(P, 1) * 60, dtype=torch.int8, device=y.device)
+    for (yy, xx, w) in ((delta, wd.x[t.h_in], p.key_buffer), (y, delta, p.value_buffer)):
+        dispatch_sgmm(yy, xx, w, p.a_start, p.a_len, p.a_loc, wd.ids, t.slot, p.a_scaling, oc, rc, li, st,
+                      tmp, P, 64, 32, 32, 32, 32, 32)
+    return y
+
+
+def run_prefill(wd, name):
+    from valora_amd.lora_prefill import lora_get_qkvo_fwd_expand, lora_get_qkvo_fwd_shrink
+    t = wd.target(name); p = t.pool
+    R = max_rank(wd)
+    y = wd.y0[name].clone()
+    delta = torch.zeros(wd.T, R, dtype=wd.dtype, device=y.device)
+    mx = int(wd.b_seq_len.max().item())
+    lora_get_qkvo_fwd_shrink(wd.x[t.h_in], p.key_buffer.view(-1, t.h_in), delta, p.a_loc, p.a_start, p.a_len,
+                             wd.b_start_loc, wd.b_seq_len, wd.req_bins, t.h_in, t.slot, R, mx)
+    lora_get_qkvo_fwd_expand(delta, p.value_buffer.view(-1, t.h_out), y, p.a_scaling, p.a_loc, p.a_start,
+                             p.a_len, wd.b_start_loc, wd.b_seq_len, wd.req_bins, t.h_out, t.slot, R, mx)
+    return y
+
+
+def assert_parity(got, want, what=""):
+    ma, rl = O.max_abs(got, want), O.rel_l2(got, want)
+    assert ma <= MAX_ABS and rl <= REL_L2, f"{what}: max_abs={ma:.3e} rel_l2={rl:.3e}"
+    return ma, rl

@@ -1,0 +1,94 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header declares,
+its size queries and argument validation work without a GPU, and the Python shims reject what
+the reference's extensions reject (valora/csrc/lora_ops.cc:79-98,124-125)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from valora_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "mlora.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mlora_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = _lib.lib()
+    names = _declared()
+    assert len(names) >= 17
+    for n in names:
+        assert hasattr(L, n), n
+    assert sorted(_lib.SYMBOLS) == names
+    assert L.mlora_version() >= 100
+
+
+def test_size_queries():
+    L = _lib.lib()
+    assert L.mlora_plan_bytes(0, 0) > 0
+    assert L.mlora_plan_bytes(256, 64) >= (32 + 3 * 256 + 2 * 8 * (16 + 64) + 4 * 64) * 4
+    assert L.mlora_partial_bytes(256, 16, 8) == 8 * 256 * 16 * 4
+    assert L.mlora_partial_bytes(10, 8, 1) == 10 * 16 * 4       # rows padded to 16 columns
+    assert L.mlora_workspace_bytes(256, 64, 16) > L.mlora_plan_bytes(256, 64)
+    assert L.mlora_plan_bytes(-1, 3) == 0
+
+
+def test_argument_validation_needs_no_gpu():
+    L = _lib.lib()
+    plan = _lib.Plan(None, 0, 0, 0, 0, 0)
+    assert L.mlora_build_plan(None, plan, None, 4, None, None, 0, 4, 0, 0) == -1
+    assert b"plan buffer is null" in L.mlora_last_error()
+    buf = ctypes.create_string_buffer(1 << 16)
+    addr = (ctypes.addressof(buf) + 255) & ~255
+    plan = _lib.Plan(addr, 64, 0, 0, 0, 0)
+    ids = (ctypes.c_int64 * 4)()
+    a = (ctypes.c_int64 * 2)()
+    rc = L.mlora_build_plan(None, plan, ctypes.addressof(ids), 4, ctypes.addressof(a), ctypes.addressof(a), 2, 4, 16, 32)
+    assert rc == -3 and b"plan buffer has 64 bytes" in L.mlora_last_error()
+    plan = _lib.Plan(addr, 1 << 15, 0, 0, 0, 0)
+    rc = L.mlora_build_plan(None, plan, ctypes.addressof(ids), 4, ctypes.addressof(a), ctypes.addressof(a), 2, 4, 48, 32)
+    assert rc == -2 and b"bm_shrink=48" in L.mlora_last_error()
+    rc = L.mlora_build_plan(None, plan, ctypes.addressof(ids), 4, ctypes.addressof(a), ctypes.addressof(a), 9000, 4, 16, 32)
+    assert rc == -2 and b"n_adapters=9000" in L.mlora_last_error()
+    # dims outside what any kernel handles -> the reference's message shape
+    pool = _lib.Pool(addr, 8, ctypes.addressof(a), ctypes.addressof(a), ctypes.addressof(a), 2, 2, 4)
+    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 0, addr, 4, 70000, 16, 0, addr, 1 << 15)
+    assert rc == -2 and L.mlora_last_error().startswith(b"No suitable kernel. h_in=70000 h_out=16 dtype=Half")
+    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 0, addr, 4, 4096, 12, 1, addr, 1 << 15)
+    assert rc == -2 and b"dtype=BFloat16" in L.mlora_last_error()
+    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 0, addr, 4, 4096, 16, 7, addr, 1 << 15)
+    assert rc == -2
+    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 5, addr, 4, 4096, 16, 0, addr, 1 << 15)
+    assert rc == -1 and b"qkvo=5" in L.mlora_last_error()
+
+
+def test_shim_rejects_what_the_reference_rejects():
+    from valora_amd.kernels import dispatch_bgmv
+    y = torch.zeros(4, 16, dtype=torch.float16)
+    x = torch.zeros(4, 64, dtype=torch.float16)
+    w = torch.zeros(8, 2, 32, dtype=torch.float16)
+    i64 = torch.zeros(4, dtype=torch.long)
+    with pytest.raises(RuntimeError, match="y must be a CUDA tensor"):
+        dispatch_bgmv(y, x, w, i64, i64, i64, i64, 0, y)
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libmlora.so")
+    with pytest.raises(RuntimeError, match="no fallback"):
+        _lib.lib()
+
+
+def test_tile_table_lookup_and_fallback():
+    from valora_amd import tile_table as tt
+    cfg = tt.lookup(256, 16, 4096, 64)
+    assert cfg.bm_shrink in (16, 32, 64) and 1 <= cfg.ksplit <= 64 and cfg.bm_expand % 16 == 0
+    fb = tt.fallback(100000, 128, 4096, 4)
+    assert fb.bm_shrink <= 32 and fb.ksplit >= 1
+    assert tt.key(300, 16, 4096, 64) == "1024:16:4096:128"

@@ -1,0 +1,192 @@
+"""GPU parity of the op entry points against the CPU oracle, always through the C ABI.
+
+Tolerance (stated by the benchmark definition): max-abs error <= 2e-2 and relative L2 error
+<= 1e-3 against the reference semantics with fp32 accumulation."""
+import pytest
+import torch
+
+from oracle import lora_oracle as O
+from valora_amd import workloads as W
+from tests._util import MAX_ABS, REL_L2, assert_parity, max_rank
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(seed, T, h_in, h_out, ranks, dtype, paged=True, id_style="random", scal=None):
+    g = torch.Generator().manual_seed(seed)
+    pool = W.make_pool(list(ranks), h_in, h_out, dtype, g, paged, std=0.05, scalings=scal)
+    A = len(ranks)
+    if id_style == "random":
+        ids = torch.randint(0, A, (T,), generator=g)
+    elif id_style == "runs":
+        ids = torch.repeat_interleave(torch.randint(0, A, (T,), generator=g),
+                                      torch.randint(1, 70, (T,), generator=g))[:T]
+    else:
+        ids = torch.randint(-1, A + 1, (T,), generator=g)
+    x = torch.randn(T, h_in, generator=g).to(dtype)
+    y0 = torch.randn(T, h_out, generator=g).to(dtype)
+    R = max(ranks)
+    v = torch.randn(T, R, generator=g).to(dtype)
+    return pool, ids, x, y0, v, R
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("T,h,ranks,ids_style", [
+    (128, 1024, (8, 16), "runs"),            # the reference's own test shape
+    (1, 4096, (16,), "random"),
+    (37, 4096, (8, 16, 32, 64), "random"),
+    (300, 3328, (16, 32, 64), "random"),     # hidden size of the reference's op bench
+    (77, 1000, (16, 8, 24), "random"),       # h % r != 0: rank groups straddle pool rows
+    (50, 11008, (64, 8), "runs"),
+    (200, 768, (128, 64, 8), "random"),      # rank 128
+    (90, 2048, (8, 16, 32), "holes"),        # ids outside [0, A): rows must stay untouched
+])
+def test_dispatch_bgmv_shrink_and_expand(dev, dtype, T, h, ranks, ids_style):
+    from valora_amd.kernels import dispatch_bgmv
+    pool, ids, x, y0, v, R = _case(T + h, T, h, h, ranks, dtype, True, ids_style,
+                                   [0.5 + 0.25 * i for i in range(len(ranks))])
+    pd = pool.to(dev)
+    for slot in (0, 3):
+        # shrink into a buffer pre-filled with a sentinel: columns >= r and skipped rows keep it
+        delta0 = torch.full((T, R), 3.0, dtype=dtype)
+        delta = delta0.to(dev)
+        dispatch_bgmv(delta, x.to(dev), pd.key_buffer, pd.a_start, pd.a_len, pd.a_loc, ids.to(dev), slot, pd.a_scaling)
+        want = O.bgmv_shrink(delta0, x, pool.key_buffer, pool.a_start, pool.a_len, pool.a_loc,
+                             torch.where((ids >= 0) & (ids < len(ranks)), ids, torch.full_like(ids, -1)), slot)
+        assert_parity(delta.cpu(), want, f"shrink slot {slot}")
+        untouched = want == 3.0
+        assert torch.equal(delta.cpu()[untouched], want[untouched])
+        y = y0.to(dev)
+        dispatch_bgmv(y, v.to(dev), pd.value_buffer, pd.a_start, pd.a_len, pd.a_loc, ids.to(dev), slot, pd.a_scaling)
+        want = O.bgmv_expand(y0, v, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc,
+                             torch.where((ids >= 0) & (ids < len(ranks)), ids, torch.full_like(ids, -1)), slot,
+                             pool.a_scaling)
+        assert_parity(y.cpu(), want, f"expand slot {slot}")
+        skipped = ~((ids >= 0) & (ids < len(ranks)))
+        assert torch.equal(y.cpu()[skipped], y0[skipped])
+
+
+def test_reference_scratch_narrower_than_rank(dev):
+    """An adapter whose rank exceeds the scratch width only contributes its first columns
+    (grid.x = feat_out in the shrink, tx = feat_in / 8 lanes in the expand)."""
+    from valora_amd.kernels import dispatch_bgmv
+    dtype = torch.float16
+    pool, ids, x, y0, v, R = _case(5, 40, 512, 512, (8, 32), dtype)
+    pd = pool.to(dev)
+    delta0 = torch.full((40, 8), 2.0, dtype=dtype)
+    delta = delta0.to(dev)
+    dispatch_bgmv(delta, x.to(dev), pd.key_buffer, pd.a_start, pd.a_len, pd.a_loc, ids.to(dev), 1, pd.a_scaling)
+    full = O.bgmv_shrink(torch.zeros(40, 32, dtype=dtype), x, pool.key_buffer, pool.a_start, pool.a_len,
+                         pool.a_loc, ids, 1)
+    assert_parity(delta.cpu(), full[:, :8], "narrow shrink")
+
+
+def test_views_and_pool_aliasing(dev):
+    """Row-sliced views (q[delora_tk_index:]) and y living in the same allocation as the pool
+    (decode writes k/v rows of the KV pool that also holds the adapters)."""
+    from valora_amd.kernels import dispatch_bgmv
+    dtype = torch.float16
+    pool, ids, x, y0, v, R = _case(9, 64, 1024, 1024, (16, 8), dtype)
+    pd = pool.to(dev)
+    n = pool.n_rows
+    big = torch.zeros(n + 64, 32, 32, dtype=dtype, device=dev)     # pool rows then 64 "KV" rows
+    big[:n] = pd.value_buffer
+    big[n:] = y0.to(dev).view(64, 32, 32)
+    yview = big[n:].view(64, 1024)[8:]                              # skip 8 rows, still contiguous
+    dispatch_bgmv(yview, v.to(dev)[8:], big, pd.a_start, pd.a_len, pd.a_loc, ids.to(dev)[8:], 2, pd.a_scaling)
+    want = O.bgmv_expand(y0[8:], v[8:], pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids[8:], 2,
+                         pool.a_scaling)
+    assert_parity(yview.cpu(), want, "aliased expand")
+    assert torch.equal(big[n:].view(64, 1024)[:8].cpu(), y0[:8])
+    assert torch.equal(big[:n].cpu(), pool.value_buffer)
+
+
+def test_error_behaviour(dev):
+    from valora_amd.kernels import dispatch_bgmv
+    dtype = torch.float16
+    pool, ids, x, y0, v, R = _case(2, 16, 512, 512, (8,), dtype)
+    pd = pool.to(dev)
+    args = (pd.a_start, pd.a_len, pd.a_loc)
+    d = torch.zeros(16, 8, dtype=dtype, device=dev)
+    with pytest.raises(RuntimeError, match="CHECK_EQ\\(indicies.size\\(0\\), x.size\\(0\\)\\)"):
+        dispatch_bgmv(d, x.to(dev), pd.key_buffer, *args, ids.to(dev)[:5], 0, pd.a_scaling)
+    with pytest.raises(RuntimeError, match="x must be contiguous"):
+        dispatch_bgmv(d, x.to(dev).t().contiguous().t(), pd.key_buffer, *args, ids.to(dev), 0, pd.a_scaling)
+    with pytest.raises(RuntimeError, match="w must be a 3D tensor"):
+        dispatch_bgmv(d, x.to(dev), pd.key_buffer.view(-1, 512), *args, ids.to(dev), 0, pd.a_scaling)
+    with pytest.raises(RuntimeError, match="No suitable kernel"):
+        dispatch_bgmv(d.float(), x.to(dev).float(), pd.key_buffer.float(), *args, ids.to(dev), 0, pd.a_scaling)
+    with pytest.raises(RuntimeError, match="No suitable kernel. h_in=512 h_out=12"):
+        dispatch_bgmv(torch.zeros(16, 12, dtype=dtype, device=dev), x.to(dev), pd.key_buffer, *args,
+                      ids.to(dev), 0, pd.a_scaling)
+    with pytest.raises(RuntimeError, match="expected scalar type Long"):
+        dispatch_bgmv(d, x.to(dev), pd.key_buffer, *args, ids.to(dev).int(), 0, pd.a_scaling)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_sgmm_and_prefill_entry_points(dev, dtype):
+    """ATMM-signature and Triton-signature entry points on a ragged batch: covered rows match the
+    oracle, rows outside the given problems / beyond max_input_len are untouched."""
+    from valora_amd.atmm_ops import dispatch_bgmv as dispatch_sgmm, shrink_accumulate
+    from valora_amd.lora_prefill import lora_get_qkvo_fwd_expand, lora_get_qkvo_fwd_shrink
+    g = torch.Generator().manual_seed(77)
+    ranks = [8, 16, 32, 16]
+    h = 512
+    pool = W.make_pool(ranks, h, h, dtype, g, True, std=0.05, scalings=[1.0, 0.5, 2.0, 1.5])
+    seq = torch.tensor([40, 3, 70, 1, 1, 33, 64], dtype=torch.int32)
+    req = torch.tensor([2, 2, 0, 1, 1, 3, 0])
+    start = (torch.cumsum(seq, 0) - seq).to(torch.int32)
+    ids = torch.repeat_interleave(req, seq.long())
+    T, R = int(ids.numel()), 32
+    x = torch.randn(T, h, generator=g).to(dtype)
+    y0 = torch.randn(T, h, generator=g).to(dtype)
+    v = torch.randn(T, R, generator=g).to(dtype)
+    pd = pool.to(dev)
+    idx = (pool.a_start, pool.a_len, pool.a_loc)
+    idxd = (pd.a_start, pd.a_len, pd.a_loc)
+    # --- ATMM signature: only the first P problems
+    oc, rc, li, st = O.count_consecutive_requests(pool.a_len, ids)
+    for P in (len(oc), 3, 0):
+        t = lambda l: torch.tensor(l + [1] * 4, dtype=torch.long, device=dev)
+        tmp = torch.zeros(60 * 8, dtype=torch.int8, device=dev)
+        d0 = torch.full((T, R), 1.5, dtype=dtype)
+        d = d0.to(dev)
+        dispatch_sgmm(d, x.to(dev), pd.key_buffer, *idxd, ids.to(dev), 1, pd.a_scaling, t(oc), t(rc), t(li), t(st),
+                      tmp, P, 64, 32, 32, 32, 32, 32)
+        want = O.sgmm_canonical(d0, x, pool.key_buffer, *idx, ids, 1, pool.a_scaling, oc, st, P)
+        assert_parity(d.cpu(), want, f"sgmm shrink P={P}")
+        y = y0.to(dev)
+        dispatch_sgmm(y, v.to(dev), pd.value_buffer, *idxd, ids.to(dev), 1, pd.a_scaling, t(oc), t(rc), t(li), t(st),
+                      tmp, P, 64, 64, 32, 64, 64, 32)
+        want = O.sgmm_canonical(y0, v, pool.value_buffer, *idx, ids, 1, pool.a_scaling, oc, st, P)
+        assert_parity(y.cpu(), want, f"sgmm expand P={P}")
+        covered = sum(oc[:P])
+        assert torch.equal(y.cpu()[covered:], y0[covered:])
+    # beta = 1 on the shrink (ATMM's accumulate)
+    shrink_accumulate(True)
+    try:
+        d0 = torch.randn(T, R, generator=g).to(dtype)
+        d = d0.to(dev)
+        dispatch_sgmm(d, x.to(dev), pd.key_buffer, *idxd, ids.to(dev), 0, pd.a_scaling, t(oc), t(rc), t(li), t(st),
+                      tmp, len(oc), 64, 32, 32, 32, 32, 32)
+        fresh = O.bgmv_shrink(torch.zeros(T, R, dtype=torch.float32), x.float(), pool.key_buffer.float(), *idx, ids, 0)
+        want = (d0.float() + fresh).to(dtype)
+        assert_parity(d.cpu(), want, "sgmm accumulate")
+    finally:
+        shrink_accumulate(False)
+    # --- Triton signature; max_input_len = 40 leaves the tails of the 70- and 64-row requests alone
+    for mx in (int(seq.max()), 40):
+        o0 = torch.full((T, R), 2.5, dtype=dtype)
+        o = o0.to(dev)
+        lora_get_qkvo_fwd_shrink(x.to(dev), pd.key_buffer.view(-1, h), o, pd.a_loc, pd.a_start, pd.a_len,
+                                 start.to(dev), seq.to(dev), req.to(dev), h, 2, R, mx)
+        want = O.triton_shrink(x, pool.key_buffer.view(-1, h), o0, pool.a_loc, pool.a_start, pool.a_len, start, seq,
+                               req, h, 2, R, mx)
+        assert_parity(o.cpu(), want, f"prefill shrink mx={mx}")
+        assert torch.equal(o.cpu() == 2.5, want == 2.5)
+        y = y0.to(dev)
+        lora_get_qkvo_fwd_expand(v.to(dev), pd.value_buffer.view(-1, h), y, pd.a_scaling, pd.a_loc, pd.a_start,
+                                 pd.a_len, start.to(dev), seq.to(dev), req.to(dev), h, 2, R, mx)
+        want = O.triton_expand(v, pool.value_buffer.view(-1, h), y0, pool.a_scaling, pool.a_loc, pool.a_start,
+                               pool.a_len, start, seq, req, h, 2, R, mx)
+        assert_parity(y.cpu(), want, f"prefill expand mx={mx}")

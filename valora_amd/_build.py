@@ -1,0 +1,54 @@
+"""Build recipe of ``libmlora.so`` (the HIP kernels + C ABI) for gfx950.
+
+``hipcc`` cross-compiles without a GPU, so this runs anywhere the ROCm toolchain is installed.
+The library is built in-tree (``valora_amd/libmlora.so``) and links only against the HIP
+runtime -- no torch, no pybind.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+from typing import List
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+SOURCES = ["api.hip", "plan.hip", "shrink.hip", "expand.hip"]
+LIB_PATH = os.path.join(HERE, "libmlora.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: the ROCm toolchain is required to build libmlora.so")
+    return exe
+
+
+def command() -> List[str]:
+    return ([hipcc()] + HIPCC_FLAGS +
+            ["-I", os.path.join(ROOT, "include"), "-I", CSRC] +
+            [os.path.join(CSRC, s) for s in SOURCES] +
+            ["-Wl,-rpath,/opt/rocm/lib", "-o", LIB_PATH])
+
+
+def build(verbose: bool = False) -> str:
+    cmd = command()
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    # the host pass warns that it does not know the packed-fp32 feature; that is expected
+    err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + err)
+    if verbose and err.strip():
+        print(err)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

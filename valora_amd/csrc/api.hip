@@ -1,0 +1,436 @@
+// C ABI of libmlora: argument validation, workspace carving and kernel dispatch.
+// The checks mirror the reference's host-side checks (valora/csrc/lora_ops.cc:79-98,124-125);
+// failures come back as a status code plus a thread-local message instead of a C++ exception.
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "mlora_internal.h"
+
+namespace mlora {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MLORA_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return MLORA_OK;
+}
+
+int expand_bn();
+
+namespace {
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+const char *dtype_name(mlora_dtype dt) { return dt == MLORA_F16 ? "Half" : "BFloat16"; }
+
+int check_dtype(mlora_dtype dt, int64_t h_in, int64_t h_out) {
+  if (dt != MLORA_F16 && dt != MLORA_BF16)
+    return fail(MLORA_ERR_NO_KERNEL, "No suitable kernel. h_in=%lld h_out=%lld dtype=%d", (long long)h_in,
+                (long long)h_out, (int)dt);
+  return MLORA_OK;
+}
+
+int check_pool(const mlora_pool *pool, const char *who) {
+  if (!pool) return fail(MLORA_ERR_INVALID, "%s: pool is null", who);
+  if (pool->n_adapters < 0 || pool->a_loc_len < 0 || pool->w_rows < 0)
+    return fail(MLORA_ERR_INVALID, "%s: negative pool size", who);
+  if (pool->n_adapters > 0 && (!pool->a_start || !pool->a_len))
+    return fail(MLORA_ERR_INVALID, "%s: a_start / a_len is null", who);
+  if (pool->a_loc_len > 0 && !pool->a_loc) return fail(MLORA_ERR_INVALID, "%s: a_loc is null", who);
+  if (pool->w_rows > 0 && !pool->w) return fail(MLORA_ERR_INVALID, "%s: w is null", who);
+  if (!aligned16(pool->w)) return fail(MLORA_ERR_INVALID, "%s: w must be 16-byte aligned", who);
+  if (pool->n_slots < 1) return fail(MLORA_ERR_INVALID, "%s: n_slots must be >= 1", who);
+  if (pool->n_adapters > MAX_ADAPTERS)
+    return fail(MLORA_ERR_NO_KERNEL, "%s: more than %lld adapters", who, (long long)MAX_ADAPTERS);
+  return MLORA_OK;
+}
+
+int check_plan(const mlora_plan *plan, int64_t T, const char *who) {
+  if (!plan || !plan->dev) return fail(MLORA_ERR_INVALID, "%s: plan is null", who);
+  if (plan->T != T) return fail(MLORA_ERR_INVALID, "%s: plan was built for T=%lld, call has T=%lld", who,
+                                (long long)plan->T, (long long)T);
+  if (plan->bytes < (size_t)plan_layout(plan->T, plan->n_adapters).total_words * 4)
+    return fail(MLORA_ERR_WORKSPACE, "%s: plan buffer too small", who);
+  return MLORA_OK;
+}
+
+// narrow (rank / scratch) and wide dims as the reference's compiled table bounds them:
+// dims < 65536 (valora/csrc/lora_ops.cc:98), 16-byte vectors (bgmv_impl.cuh:166-168).
+int check_dims(int64_t T, int64_t wide, int64_t narrow, int64_t h_in, int64_t h_out, mlora_dtype dt) {
+  if (T < 0 || T > MAX_TOKENS) return fail(MLORA_ERR_INVALID, "T=%lld out of range", (long long)T);
+  if (wide <= 0 || wide >= 65536 || narrow <= 0 || narrow > MAX_RANK || (wide % 8) != 0 || (narrow % 8) != 0)
+    return fail(MLORA_ERR_NO_KERNEL, "No suitable kernel. h_in=%lld h_out=%lld dtype=%s", (long long)h_in,
+                (long long)h_out, dtype_name(dt));
+  return MLORA_OK;
+}
+
+int default_bm_shrink(int64_t T, int64_t A) {
+  (void)A;
+  return T <= 2048 ? 16 : T <= 8192 ? 32 : 64;
+}
+int default_bm_expand(int64_t T, int64_t A) {
+  (void)A;
+  return T <= 1024 ? 32 : T <= 8192 ? 64 : 128;
+}
+int default_ksplit(int64_t T, int64_t A, int bm, int64_t h_in) {
+  // aim for >= ~1024 workgroups, keep >= 256 K elements per workgroup, at most 16 partials
+  int64_t tiles = tiles_upper(T, A, bm);
+  if (tiles > T) tiles = T;
+  if (tiles < 1) tiles = 1;
+  int64_t ks = (1024 + tiles - 1) / tiles;
+  int64_t kmax = h_in / 256;
+  if (kmax < 1) kmax = 1;
+  if (ks > kmax) ks = kmax;
+  if (ks > 16) ks = 16;
+  if (ks < 1) ks = 1;
+  return (int)ks;
+}
+
+PoolDev pool_dev(const mlora_pool *p) {
+  PoolDev d;
+  d.w = static_cast<const uint16_t *>(p->w);
+  d.w_rows = p->w_rows;
+  d.a_loc = p->a_loc;
+  d.a_loc_len = p->a_loc_len;
+  return d;
+}
+
+struct Carver {
+  char *p;
+  size_t left;
+  void *take(size_t n) {
+    n = (n + 255) & ~(size_t)255;
+    if (n > left) return nullptr;
+    void *r = p;
+    p += n;
+    left -= n;
+    return r;
+  }
+};
+
+}  // namespace
+}  // namespace mlora
+
+using namespace mlora;
+
+extern "C" {
+
+const char *mlora_last_error(void) { return g_err; }
+int mlora_version(void) { return 100; }
+
+size_t mlora_plan_bytes(int64_t T, int64_t n_adapters) {
+  if (T < 0 || n_adapters < 0) return 0;
+  return (size_t)plan_layout(T, n_adapters).total_words * 4;
+}
+
+size_t mlora_partial_bytes(int64_t T, int64_t max_rank, int32_t ksplit) {
+  if (T < 0 || max_rank < 0 || ksplit < 1) return 0;
+  size_t n = (size_t)ksplit * (size_t)T * (size_t)partial_stride(max_rank) * 4;
+  return n < 256 ? 256 : n;
+}
+
+size_t mlora_workspace_bytes(int64_t T, int64_t n_adapters, int64_t max_rank) {
+  if (T < 0 || n_adapters < 0 || max_rank < 0) return 0;
+  auto up = [](size_t n) { return (n + 255) & ~(size_t)255; };
+  const int ks = default_ksplit(T, n_adapters, default_bm_shrink(T, n_adapters), 1 << 16);
+  return up(mlora_plan_bytes(T, n_adapters)) + up(mlora_partial_bytes(T, max_rank, ks)) +
+         up((size_t)T * 8 + 8) + 256;
+}
+
+int mlora_build_plan(void *stream, mlora_plan *plan, const int64_t *ids, int64_t T, const int64_t *a_start,
+                     const int64_t *a_len, int64_t n_adapters, int32_t n_slots, int32_t bm_shrink,
+                     int32_t bm_expand) {
+  if (!plan || !plan->dev) return fail(MLORA_ERR_INVALID, "build_plan: plan buffer is null");
+  if (T < 0 || T > MAX_TOKENS) return fail(MLORA_ERR_INVALID, "build_plan: T=%lld out of range", (long long)T);
+  if (n_adapters < 0 || n_adapters > MAX_ADAPTERS)
+    return fail(MLORA_ERR_NO_KERNEL, "build_plan: n_adapters=%lld out of range (max %lld)", (long long)n_adapters,
+                (long long)MAX_ADAPTERS);
+  if (T > 0 && !ids) return fail(MLORA_ERR_INVALID, "build_plan: ids is null");
+  if (n_adapters > 0 && (!a_start || !a_len)) return fail(MLORA_ERR_INVALID, "build_plan: a_start / a_len is null");
+  if (n_slots < 1) return fail(MLORA_ERR_INVALID, "build_plan: n_slots must be >= 1");
+  if (bm_shrink == 0) bm_shrink = default_bm_shrink(T, n_adapters);
+  if (bm_expand == 0) bm_expand = default_bm_expand(T, n_adapters);
+  if (bm_shrink != 16 && bm_shrink != 32 && bm_shrink != 64)
+    return fail(MLORA_ERR_NO_KERNEL, "build_plan: bm_shrink=%d not in {16,32,64}", bm_shrink);
+  if (bm_expand < 16 || bm_expand > 256 || (bm_expand % 16) != 0)
+    return fail(MLORA_ERR_NO_KERNEL, "build_plan: bm_expand=%d not a multiple of 16 in [16,256]", bm_expand);
+  const PlanLayout L = plan_layout(T, n_adapters);
+  if (plan->bytes < (size_t)L.total_words * 4)
+    return fail(MLORA_ERR_WORKSPACE, "build_plan: plan buffer has %zu bytes, needs %zu", plan->bytes,
+                (size_t)L.total_words * 4);
+  if (!aligned16(plan->dev)) return fail(MLORA_ERR_INVALID, "build_plan: plan buffer must be 16-byte aligned");
+  plan->T = T;
+  plan->n_adapters = n_adapters;
+  plan->bm_shrink = bm_shrink;
+  plan->bm_expand = bm_expand;
+  return launch_plan((hipStream_t)stream, static_cast<int32_t *>(plan->dev), L, ids, a_start, a_len, n_slots,
+                     bm_shrink, bm_expand);
+}
+
+int mlora_count_consecutive(void *stream, const int64_t *lora_rank, int64_t n_adapters, const int64_t *indicies,
+                            int64_t T, int64_t *output_counts, int64_t *rank_counts, int64_t *lora_ids,
+                            int64_t *start_ids, int64_t *num_runs) {
+  if (T < 0 || T > MAX_TOKENS) return fail(MLORA_ERR_INVALID, "count_consecutive: T=%lld out of range", (long long)T);
+  if (!num_runs) return fail(MLORA_ERR_INVALID, "count_consecutive: num_runs is null");
+  if (T > 0 && (!indicies || !output_counts || !rank_counts || !lora_ids || !start_ids || !lora_rank))
+    return fail(MLORA_ERR_INVALID, "count_consecutive: null pointer");
+  return launch_count_consecutive((hipStream_t)stream, lora_rank, n_adapters, indicies, T, output_counts,
+                                  rank_counts, lora_ids, start_ids, num_runs);
+}
+
+int mlora_ids_from_segments(void *stream, int64_t *ids_out, const int64_t *ids_in, const int64_t *start_ids,
+                            const int64_t *output_counts, int64_t P, int64_t T) {
+  if (T < 0 || P < 0) return fail(MLORA_ERR_INVALID, "ids_from_segments: negative size");
+  if (T > 0 && (!ids_out || !ids_in)) return fail(MLORA_ERR_INVALID, "ids_from_segments: null pointer");
+  if (P > 0 && (!start_ids || !output_counts)) return fail(MLORA_ERR_INVALID, "ids_from_segments: null segments");
+  return launch_ids_from_segments((hipStream_t)stream, ids_out, ids_in, start_ids, output_counts, P, T);
+}
+
+int mlora_ids_from_requests(void *stream, int64_t *ids_out, const int32_t *b_start_loc, const int32_t *b_seq_len,
+                            const int64_t *b_indicies, int64_t n_req, int64_t T, int64_t max_rows) {
+  if (T < 0 || n_req < 0) return fail(MLORA_ERR_INVALID, "ids_from_requests: negative size");
+  if (T > 0 && !ids_out) return fail(MLORA_ERR_INVALID, "ids_from_requests: null pointer");
+  if (n_req > 0 && (!b_start_loc || !b_seq_len || !b_indicies))
+    return fail(MLORA_ERR_INVALID, "ids_from_requests: null request operands");
+  return launch_ids_from_requests((hipStream_t)stream, ids_out, b_start_loc, b_seq_len, b_indicies, n_req, T,
+                                  max_rows);
+}
+
+int mlora_shrink_partial(void *stream, const mlora_plan *plan, float *partial, size_t partial_bytes, const void *x,
+                         int64_t T, int64_t h_in, int64_t max_rank, const mlora_pool *pool, int32_t slot,
+                         int32_t ksplit, mlora_dtype dtype) {
+  if (int rc = check_dtype(dtype, h_in, max_rank)) return rc;
+  if (int rc = check_dims(T, h_in, max_rank, h_in, max_rank, dtype)) return rc;
+  if (int rc = check_plan(plan, T, "shrink")) return rc;
+  if (int rc = check_pool(pool, "shrink")) return rc;
+  if (T == 0) return MLORA_OK;
+  if (!x || !partial) return fail(MLORA_ERR_INVALID, "shrink: null pointer");
+  if (!aligned16(x) || !aligned16(partial)) return fail(MLORA_ERR_INVALID, "shrink: x and partial must be 16-byte aligned");
+  if (slot < 0 || slot >= pool->n_slots) return fail(MLORA_ERR_INVALID, "shrink: slot %d outside [0,%d)", slot, pool->n_slots);
+  if (ksplit < 1 || ksplit > 64) return fail(MLORA_ERR_INVALID, "shrink: ksplit=%d outside [1,64]", ksplit);
+  if (partial_bytes < mlora_partial_bytes(T, max_rank, ksplit))
+    return fail(MLORA_ERR_WORKSPACE, "shrink: partial buffer has %zu bytes, needs %zu", partial_bytes,
+                mlora_partial_bytes(T, max_rank, ksplit));
+  const PlanLayout L = plan_layout(plan->T, plan->n_adapters);
+  ShrinkArgs a;
+  a.plan = static_cast<const int32_t *>(plan->dev);
+  a.off_perm = L.off_perm;
+  a.off_tiles = L.off_tiles_s;
+  a.partial = partial;
+  a.x = static_cast<const uint16_t *>(x);
+  a.pool = pool_dev(pool);
+  a.T = (int)T;
+  a.h_in = (int)h_in;
+  a.rp = (int)partial_stride(max_rank);
+  a.slot = slot;
+  a.ksplit = ksplit;
+  a.kchunk = (int)align_up((h_in + ksplit - 1) / ksplit, 128);
+  return launch_shrink((hipStream_t)stream, a, plan->bm_shrink, (int)max_rank,
+                       tiles_upper(T, plan->n_adapters, plan->bm_shrink), dtype);
+}
+
+int mlora_shrink_finish(void *stream, const mlora_plan *plan, const float *partial, void *y, int64_t T,
+                        int64_t y_stride, int64_t max_rank, int32_t ksplit, int32_t mode, int32_t width,
+                        mlora_dtype dtype) {
+  if (int rc = check_dtype(dtype, 0, max_rank)) return rc;
+  if (int rc = check_plan(plan, T, "shrink_finish")) return rc;
+  if (T == 0) return MLORA_OK;
+  if (!partial || !y) return fail(MLORA_ERR_INVALID, "shrink_finish: null pointer");
+  if (mode < 0 || mode > 2) return fail(MLORA_ERR_INVALID, "shrink_finish: bad mode %d", mode);
+  if (max_rank <= 0 || max_rank > MAX_RANK) return fail(MLORA_ERR_NO_KERNEL, "shrink_finish: max_rank=%lld", (long long)max_rank);
+  if (y_stride < 1 || (mode == MLORA_SHRINK_ZERO_PAD && width > y_stride))
+    return fail(MLORA_ERR_INVALID, "shrink_finish: width %d exceeds row stride %lld", width, (long long)y_stride);
+  const PlanLayout L = plan_layout(plan->T, plan->n_adapters);
+  FinishArgs a;
+  a.plan = static_cast<const int32_t *>(plan->dev);
+  a.off_perm = L.off_perm;
+  a.off_prank = L.off_prank;
+  a.partial = partial;
+  a.y = static_cast<uint16_t *>(y);
+  a.y_stride = y_stride;
+  a.T = (int)T;
+  a.rp = (int)partial_stride(max_rank);
+  a.ncols = (int)(max_rank < y_stride ? max_rank : y_stride);
+  a.ksplit = ksplit;
+  a.mode = mode;
+  a.width = width;
+  return launch_finish((hipStream_t)stream, a, dtype);
+}
+
+int mlora_expand(void *stream, const mlora_plan *plan, void *y, int64_t T, int64_t h_out, const float *partial,
+                 int32_t ksplit, const void *xv, int64_t v_stride, int64_t max_rank, const mlora_pool *pool,
+                 int32_t slot, const void *scales, mlora_dtype dtype) {
+  if (int rc = check_dtype(dtype, max_rank, h_out)) return rc;
+  if (int rc = check_dims(T, h_out, max_rank, max_rank, h_out, dtype)) return rc;
+  if (int rc = check_plan(plan, T, "expand")) return rc;
+  if (int rc = check_pool(pool, "expand")) return rc;
+  if (T == 0) return MLORA_OK;
+  if (!y || !scales) return fail(MLORA_ERR_INVALID, "expand: null pointer");
+  if (!partial && !xv) return fail(MLORA_ERR_INVALID, "expand: neither partial nor xv given");
+  if (!aligned16(y) || !aligned16(partial) || !aligned16(xv))
+    return fail(MLORA_ERR_INVALID, "expand: y, partial and xv must be 16-byte aligned");
+  if (!partial && (v_stride < max_rank || (v_stride % 8) != 0))
+    return fail(MLORA_ERR_NO_KERNEL, "No suitable kernel. h_in=%lld h_out=%lld dtype=%s", (long long)v_stride,
+                (long long)h_out, dtype_name(dtype));
+  if (slot < 0 || slot >= pool->n_slots) return fail(MLORA_ERR_INVALID, "expand: slot %d outside [0,%d)", slot, pool->n_slots);
+  if (partial && (ksplit < 1 || ksplit > 64)) return fail(MLORA_ERR_INVALID, "expand: ksplit=%d outside [1,64]", ksplit);
+  const PlanLayout L = plan_layout(plan->T, plan->n_adapters);
+  ExpandArgs a;
+  a.plan = static_cast<const int32_t *>(plan->dev);
+  a.off_perm = L.off_perm;
+  a.off_tiles = L.off_tiles_e;
+  a.y = static_cast<uint16_t *>(y);
+  a.partial = partial;
+  a.xv = static_cast<const uint16_t *>(xv);
+  a.v_stride = v_stride;
+  a.pool = pool_dev(pool);
+  a.scales = static_cast<const uint16_t *>(scales);
+  a.T = (int)T;
+  a.h_out = (int)h_out;
+  a.rp = (int)partial_stride(max_rank);
+  a.kmax = (int)max_rank;
+  a.slot = slot;
+  a.ksplit = ksplit;
+  a.n_ochunks = (int)((h_out + expand_bn() - 1) / expand_bn());
+  return launch_expand((hipStream_t)stream, a, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand),
+                       dtype);
+}
+
+int mlora_lora_apply(void *stream, const mlora_plan *plan, float *partial, size_t partial_bytes, void *y,
+                     const void *x, int64_t T, int64_t h_in, int64_t h_out, int64_t max_rank,
+                     const mlora_pool *pool_a, const mlora_pool *pool_b, int32_t slot, const void *scales,
+                     int32_t ksplit, mlora_dtype dtype) {
+  if (!plan) return fail(MLORA_ERR_INVALID, "lora_apply: plan is null");
+  if (ksplit == 0) ksplit = default_ksplit(T, plan->n_adapters, plan->bm_shrink, h_in);
+  if (int rc = mlora_shrink_partial(stream, plan, partial, partial_bytes, x, T, h_in, max_rank, pool_a, slot, ksplit,
+                                    dtype))
+    return rc;
+  return mlora_expand(stream, plan, y, T, h_out, partial, ksplit, nullptr, 0, max_rank, pool_b, slot, scales, dtype);
+}
+
+// ---- one-call entry points ------------------------------------------------------------------------
+
+static int one_call(void *stream, void *y, const void *x, const mlora_pool *pool, const int64_t *ids, int64_t qkvo,
+                    const void *scales, int64_t T, int64_t h_in, int64_t h_out, mlora_dtype dtype, int shrink_mode,
+                    int shrink_width, int64_t narrow_stride, Carver &ws, const char *who) {
+  if (int rc = check_pool(pool, who)) return rc;
+  if (qkvo < 0 || qkvo >= pool->n_slots) return fail(MLORA_ERR_INVALID, "%s: qkvo=%lld outside [0,%d)", who, (long long)qkvo, pool->n_slots);
+  const bool expand = h_in < h_out;  // valora/csrc/bgmv/bgmv_impl.cuh:221
+  const int64_t narrow = expand ? h_in : h_out;
+  const int64_t wide = expand ? h_out : h_in;
+  if (int rc = check_dims(T, wide, narrow, h_in, h_out, dtype)) return rc;
+  if (T == 0) return MLORA_OK;
+  mlora_plan plan;
+  plan.bytes = mlora_plan_bytes(T, pool->n_adapters);
+  plan.dev = ws.take(plan.bytes);
+  if (!plan.dev) return fail(MLORA_ERR_WORKSPACE, "%s: workspace too small (needs %zu bytes)", who,
+                             mlora_workspace_bytes(T, pool->n_adapters, narrow));
+  if (int rc = mlora_build_plan(stream, &plan, ids, T, pool->a_start, pool->a_len, pool->n_adapters, pool->n_slots, 0, 0))
+    return rc;
+  if (expand) {
+    if (narrow_stride == 0) narrow_stride = h_in;
+    return mlora_expand(stream, &plan, y, T, h_out, nullptr, 0, x, narrow_stride, narrow, pool, (int32_t)qkvo, scales,
+                        dtype);
+  }
+  const int ksplit = default_ksplit(T, pool->n_adapters, plan.bm_shrink, h_in);
+  const size_t pbytes = mlora_partial_bytes(T, narrow, ksplit);
+  float *partial = static_cast<float *>(ws.take(pbytes));
+  if (!partial) return fail(MLORA_ERR_WORKSPACE, "%s: workspace too small (needs %zu bytes)", who,
+                            mlora_workspace_bytes(T, pool->n_adapters, narrow));
+  if (int rc = mlora_shrink_partial(stream, &plan, partial, pbytes, x, T, h_in, narrow, pool, (int32_t)qkvo, ksplit, dtype))
+    return rc;
+  if (narrow_stride == 0) narrow_stride = h_out;
+  return mlora_shrink_finish(stream, &plan, partial, y, T, narrow_stride, narrow, ksplit, shrink_mode,
+                             shrink_width, dtype);
+}
+
+int mlora_dispatch_bgmv(void *stream, void *y, const void *x, const mlora_pool *pool, const int64_t *indicies,
+                        int64_t qkvo, const void *lora_scales, int64_t T, int64_t h_in, int64_t h_out,
+                        mlora_dtype dtype, void *workspace, size_t workspace_bytes) {
+  if (int rc = check_dtype(dtype, h_in, h_out)) return rc;
+  if (T > 0 && (!y || !x || !indicies)) return fail(MLORA_ERR_INVALID, "dispatch_bgmv: null pointer");
+  if (T > 0 && (!workspace || !aligned16(workspace))) return fail(MLORA_ERR_WORKSPACE, "dispatch_bgmv: workspace missing or misaligned");
+  if (T > 0 && h_in < h_out && !lora_scales) return fail(MLORA_ERR_INVALID, "dispatch_bgmv: lora_scales is null");
+  Carver ws{static_cast<char *>(workspace), workspace_bytes};
+  return one_call(stream, y, x, pool, indicies, qkvo, lora_scales, T, h_in, h_out, dtype, MLORA_SHRINK_OVERWRITE, 0, 0,
+                  ws, "dispatch_bgmv");
+}
+
+int mlora_dispatch_sgmm(void *stream, void *y, const void *x, const mlora_pool *pool, const int64_t *indicies,
+                        int64_t qkvo, const void *lora_scales, const int64_t *output_counts,
+                        const int64_t *start_ids, int64_t num_problems, int64_t T, int64_t h_in, int64_t h_out,
+                        mlora_dtype dtype, int32_t shrink_mode, void *workspace, size_t workspace_bytes) {
+  if (int rc = check_dtype(dtype, h_in, h_out)) return rc;
+  if (T < 0 || T > MAX_TOKENS) return fail(MLORA_ERR_INVALID, "dispatch_sgmm: T=%lld out of range", (long long)T);
+  if (num_problems < 0) return fail(MLORA_ERR_INVALID, "dispatch_sgmm: num_problems < 0");
+  if (shrink_mode != MLORA_SHRINK_OVERWRITE && shrink_mode != MLORA_SHRINK_ACCUMULATE)
+    return fail(MLORA_ERR_INVALID, "dispatch_sgmm: bad shrink_mode %d", shrink_mode);
+  if (T == 0) return MLORA_OK;
+  if (!y || !x || !indicies) return fail(MLORA_ERR_INVALID, "dispatch_sgmm: null pointer");
+  if (!workspace || !aligned16(workspace)) return fail(MLORA_ERR_WORKSPACE, "dispatch_sgmm: workspace missing or misaligned");
+  if (h_in < h_out && !lora_scales) return fail(MLORA_ERR_INVALID, "dispatch_sgmm: lora_scales is null");
+  Carver ws{static_cast<char *>(workspace), workspace_bytes};
+  int64_t *ids_eff = static_cast<int64_t *>(ws.take((size_t)T * 8));
+  if (!ids_eff) return fail(MLORA_ERR_WORKSPACE, "dispatch_sgmm: workspace too small");
+  if (int rc = mlora_ids_from_segments(stream, ids_eff, indicies, start_ids, output_counts, num_problems, T)) return rc;
+  return one_call(stream, y, x, pool, ids_eff, qkvo, lora_scales, T, h_in, h_out, dtype, shrink_mode, 0, 0, ws,
+                  "dispatch_sgmm");
+}
+
+int mlora_prefill_shrink(void *stream, void *o, const void *x, const mlora_pool *pool, const int32_t *b_start_loc,
+                         const int32_t *b_seq_len, const int64_t *b_indicies, int64_t n_req, int64_t T,
+                         int64_t hidden, int64_t o_stride, int64_t qkvo, int64_t max_rank, int64_t max_input_len,
+                         mlora_dtype dtype, void *workspace, size_t workspace_bytes) {
+  if (int rc = check_dtype(dtype, hidden, max_rank)) return rc;
+  if (T < 0 || T > MAX_TOKENS || n_req < 0) return fail(MLORA_ERR_INVALID, "prefill_shrink: bad size");
+  if (T == 0 || n_req == 0) return MLORA_OK;
+  if (!o || !x) return fail(MLORA_ERR_INVALID, "prefill_shrink: null pointer");
+  if (!workspace || !aligned16(workspace)) return fail(MLORA_ERR_WORKSPACE, "prefill_shrink: workspace missing or misaligned");
+  if (max_rank <= 0 || max_rank > MAX_RANK) return fail(MLORA_ERR_NO_KERNEL, "prefill_shrink: max_rank=%lld", (long long)max_rank);
+  Carver ws{static_cast<char *>(workspace), workspace_bytes};
+  int64_t *ids_eff = static_cast<int64_t *>(ws.take((size_t)T * 8));
+  if (!ids_eff) return fail(MLORA_ERR_WORKSPACE, "prefill_shrink: workspace too small");
+  // rows visited per request: grid z covers cdiv(max_input_len, 32) blocks of 32 rows (lora_prefill.py:147)
+  const int64_t max_rows = (max_input_len + 31) / 32 * 32;
+  if (int rc = mlora_ids_from_requests(stream, ids_eff, b_start_loc, b_seq_len, b_indicies, n_req, T, max_rows)) return rc;
+  // columns stored: cdiv(max_rank, BLOCK_N) blocks of BLOCK_N = 16 (or max_rank when <= 8) (lora_prefill.py:142,147)
+  const int64_t block_n = max_rank > 8 ? 16 : max_rank;
+  int64_t width = (max_rank + block_n - 1) / block_n * block_n;
+  if (width > o_stride) width = o_stride;
+  const int64_t narrow = align_up(max_rank, 8);
+  return one_call(stream, o, x, pool, ids_eff, qkvo, nullptr, T, hidden, narrow, dtype, MLORA_SHRINK_ZERO_PAD,
+                  (int)width, o_stride, ws, "prefill_shrink");
+}
+
+int mlora_prefill_expand(void *stream, void *o, const void *x, const mlora_pool *pool, const void *scale,
+                         const int32_t *b_start_loc, const int32_t *b_seq_len, const int64_t *b_indicies,
+                         int64_t n_req, int64_t T, int64_t x_stride, int64_t feat_out, int64_t qkvo,
+                         int64_t max_rank, int64_t max_input_len, mlora_dtype dtype, void *workspace,
+                         size_t workspace_bytes) {
+  if (int rc = check_dtype(dtype, max_rank, feat_out)) return rc;
+  if (T < 0 || T > MAX_TOKENS || n_req < 0) return fail(MLORA_ERR_INVALID, "prefill_expand: bad size");
+  if (T == 0 || n_req == 0) return MLORA_OK;
+  if (!o || !x || !scale) return fail(MLORA_ERR_INVALID, "prefill_expand: null pointer");
+  if (!workspace || !aligned16(workspace)) return fail(MLORA_ERR_WORKSPACE, "prefill_expand: workspace missing or misaligned");
+  if (max_rank <= 0 || max_rank > MAX_RANK || max_rank >= feat_out)
+    return fail(MLORA_ERR_NO_KERNEL, "prefill_expand: max_rank=%lld", (long long)max_rank);
+  Carver ws{static_cast<char *>(workspace), workspace_bytes};
+  int64_t *ids_eff = static_cast<int64_t *>(ws.take((size_t)T * 8));
+  if (!ids_eff) return fail(MLORA_ERR_WORKSPACE, "prefill_expand: workspace too small");
+  const int64_t max_rows = (max_input_len + 31) / 32 * 32;
+  if (int rc = mlora_ids_from_requests(stream, ids_eff, b_start_loc, b_seq_len, b_indicies, n_req, T, max_rows)) return rc;
+  return one_call(stream, o, x, pool, ids_eff, qkvo, scale, T, align_up(max_rank, 8), feat_out, dtype,
+                  MLORA_SHRINK_OVERWRITE, 0, x_stride, ws, "prefill_expand");
+}
+
+}  // extern "C"

@@ -1,0 +1,73 @@
+// Device-side helpers shared by the gfx950 LoRA kernels: 16-byte vector access and the
+// per-dtype MFMA / conversion traits.  (The reference's counterpart is the 1300-line
+// vec_dtypes.cuh, valora/csrc/bgmv/vec_dtypes.cuh:16-30,754-800; only fp16 and bf16 exist here.)
+#pragma once
+
+#include "mlora_internal.h"
+
+namespace mlora {
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+
+template <typename To, typename From>
+__device__ __forceinline__ To as(const From &v) {
+  static_assert(sizeof(To) == sizeof(From), "size mismatch");
+  return __builtin_bit_cast(To, v);
+}
+
+// One global_load_dwordx4 / global_store_dwordx4.  Addresses must be 16-byte aligned.
+__device__ __forceinline__ u32x4 load16(const uint16_t *p) { return *reinterpret_cast<const u32x4 *>(p); }
+__device__ __forceinline__ void store16(uint16_t *p, u32x4 v) { *reinterpret_cast<u32x4 *>(p) = v; }
+
+template <typename T>
+struct Traits;
+
+template <>
+struct Traits<_Float16> {
+  using vec8 = f16x8;
+  static __device__ __forceinline__ f32x4 mfma(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t h) { return (float)as<_Float16>(h); }
+  static __device__ __forceinline__ uint16_t from_float(float f) { return as<uint16_t>((_Float16)f); }
+};
+
+template <>
+struct Traits<__bf16> {
+  using vec8 = bf16x8;
+  static __device__ __forceinline__ f32x4 mfma(vec8 a, vec8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t h) { return as<float>((uint32_t)h << 16); }
+  // round to nearest even; NaN stays NaN
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    uint32_t x = as<uint32_t>(f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+    x += 0x7fffu + ((x >> 16) & 1u);
+    return (uint16_t)(x >> 16);
+  }
+};
+
+// 8 packed T values <-> 8 floats
+template <typename T>
+__device__ __forceinline__ void unpack8(u32x4 v, float (&f)[8]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = Traits<T>::to_float((uint16_t)(v[i] & 0xffffu));
+    f[2 * i + 1] = Traits<T>::to_float((uint16_t)(v[i] >> 16));
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
+  u32x4 v;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    v[i] = (uint32_t)Traits<T>::from_float(f[2 * i]) | ((uint32_t)Traits<T>::from_float(f[2 * i + 1]) << 16);
+  return v;
+}
+
+}  // namespace mlora

@@ -1,0 +1,121 @@
+// Internal declarations shared by the kernel translation units of libmlora (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mlora.h"
+
+namespace mlora {
+
+// ---- plan buffer layout (int32 words) ------------------------------------------------------
+//   hdr[32] | perm[T] | padapter[T] | prank[T] | tiles_s[max_tiles][8] | tiles_e[max_tiles][8]
+//   | scratch: cnt[A] gstart[A] toff_s[A] toff_e[A]
+// perm[p]     token index at sorted position p (tokens grouped by adapter, original order kept
+//             inside a group); positions >= hdr[H_NACTIVE] are unused
+// padapter[p] adapter of position p;  prank[p] its rank
+// tile        {adapter, rank, first position, token count, a_start[adapter], 0, 0, 0}
+constexpr int HDR_WORDS = 32;
+constexpr int TILE_WORDS = 8;
+constexpr int32_t PLAN_MAGIC = 0x4d4c5241;
+enum Hdr {
+  H_MAGIC = 0, H_T = 1, H_NADAPTERS = 2, H_NTILES_S = 3, H_NTILES_E = 4, H_NGROUPS = 5,
+  H_MAXRANK = 6, H_ERR = 7, H_BM_S = 8, H_BM_E = 9, H_NACTIVE = 10
+};
+// bits of hdr[H_ERR]
+enum PlanErr { PERR_START_OVERFLOW = 1 };
+
+constexpr int64_t MAX_ADAPTERS = 8192;   // per-wave histograms live in LDS
+constexpr int64_t MAX_TOKENS = 1 << 22;
+constexpr int MAX_RANK = 128;
+
+struct PlanLayout {
+  int64_t T, A, max_tiles;
+  int64_t off_perm, off_padapter, off_prank, off_tiles_s, off_tiles_e, off_scratch, total_words;
+};
+
+static inline __host__ __device__ int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+static inline PlanLayout plan_layout(int64_t T, int64_t A) {
+  PlanLayout L;
+  L.T = T;
+  L.A = A;
+  L.max_tiles = (T + 15) / 16 + (A < T ? A : T);
+  L.off_perm = HDR_WORDS;
+  L.off_padapter = align_up(L.off_perm + T, 8);
+  L.off_prank = align_up(L.off_padapter + T, 8);
+  L.off_tiles_s = align_up(L.off_prank + T, 8);
+  L.off_tiles_e = L.off_tiles_s + L.max_tiles * TILE_WORDS;
+  L.off_scratch = L.off_tiles_e + L.max_tiles * TILE_WORDS;
+  L.total_words = L.off_scratch + 4 * A + 8;
+  return L;
+}
+
+// upper bound of the tile count for tile height bm (what the grids are sized with)
+static inline int64_t tiles_upper(int64_t T, int64_t A, int bm) {
+  return (T + bm - 1) / bm + (A < T ? A : T);
+}
+
+static inline int64_t partial_stride(int64_t max_rank) { return align_up(max_rank, 16); }
+
+// ---- error reporting (api.hip) ---------------------------------------------------------------
+int fail(int code, const char *fmt, ...);
+int check_launch(const char *what);
+
+// ---- kernel launchers ------------------------------------------------------------------------
+struct PoolDev {
+  const uint16_t *w;
+  int64_t w_rows;
+  const int64_t *a_loc;
+  int64_t a_loc_len;
+};
+
+struct ShrinkArgs {
+  const int32_t *plan;
+  int64_t off_perm, off_tiles;
+  float *partial;
+  const uint16_t *x;
+  PoolDev pool;
+  int T, h_in, rp, slot, ksplit, kchunk;
+};
+
+struct ExpandArgs {
+  const int32_t *plan;
+  int64_t off_perm, off_tiles;
+  uint16_t *y;
+  const float *partial;
+  const uint16_t *xv;
+  int64_t v_stride;
+  PoolDev pool;
+  const uint16_t *scales;
+  int T, h_out, rp, kmax, slot, ksplit, n_ochunks;
+};
+
+struct FinishArgs {
+  const int32_t *plan;
+  int64_t off_perm, off_prank;
+  const float *partial;
+  uint16_t *y;
+  int64_t y_stride;
+  int T, rp, ncols, ksplit, mode, width;
+};
+
+int launch_plan(hipStream_t st, int32_t *plan, const PlanLayout &L, const int64_t *ids,
+                const int64_t *a_start, const int64_t *a_len, int n_slots, int bm_s, int bm_e);
+int launch_count_consecutive(hipStream_t st, const int64_t *lora_rank, int64_t n_adapters,
+                             const int64_t *indicies, int64_t T, int64_t *output_counts,
+                             int64_t *rank_counts, int64_t *lora_ids, int64_t *start_ids,
+                             int64_t *num_runs);
+int launch_ids_from_segments(hipStream_t st, int64_t *ids_out, const int64_t *ids_in,
+                             const int64_t *start_ids, const int64_t *output_counts, int64_t P,
+                             int64_t T);
+int launch_ids_from_requests(hipStream_t st, int64_t *ids_out, const int32_t *b_start_loc,
+                             const int32_t *b_seq_len, const int64_t *b_indicies, int64_t n_req,
+                             int64_t T, int64_t max_rows);
+int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int64_t grid_tiles,
+                  mlora_dtype dt);
+int launch_finish(hipStream_t st, const FinishArgs &a, mlora_dtype dt);
+int launch_expand(hipStream_t st, const ExpandArgs &a, int max_rank, int64_t grid_tiles,
+                  mlora_dtype dt);
+
+}  // namespace mlora

@@ -1,0 +1,313 @@
+// Ragged segment / adapter-index builders for gfx950.
+//
+//  * plan_kernel              stable counting sort of tokens by adapter + adapter-grouped tile
+//                             lists (what the shrink / expand kernels iterate over)
+//  * count_consecutive_kernel parallel run-length encoding, bit-exact with the reference's
+//                             single-thread count_consecutive_requests
+//                             (atmm/valora/csrc/bgmv/bgmv_impl.cuh:39-72)
+//  * ids_fill / ids_cover_*   per-token ids from segment or per-request operands
+//
+// All are single-workgroup or trivially parallel integer kernels: the inputs are a few KB and
+// the work is launch-latency bound, so one 1024-thread workgroup with LDS histograms is used
+// instead of a multi-pass device-wide sort.
+#include "mlora_internal.h"
+
+namespace mlora {
+
+namespace {
+
+constexpr int PLAN_THREADS = 1024;
+constexpr int PLAN_WAVES = PLAN_THREADS / 64;
+constexpr int HIST_WORDS = 8192;  // LDS words for the per-wave histograms
+
+__device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    int n = __shfl_up(v, d, 64);
+    if (lane >= d) v += n;
+  }
+  return v;
+}
+
+// exclusive prefix of v over the 1024 threads; *total gets the block sum.
+__device__ __forceinline__ int block_exclusive_scan(int v, int *total, int *wsum /* LDS[17] */) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int inc = wave_inclusive_scan(v, lane);
+  __syncthreads();  // wsum may still be read from a previous scan
+  if (lane == 63) wsum[wave] = inc;
+  __syncthreads();
+  if (wave == 0) {
+    int w = lane < PLAN_WAVES ? wsum[lane] : 0;
+    int winc = wave_inclusive_scan(w, lane);
+    if (lane < PLAN_WAVES) wsum[lane] = winc - w;
+    if (lane == PLAN_WAVES - 1) wsum[PLAN_WAVES] = winc;
+  }
+  __syncthreads();
+  *total = wsum[PLAN_WAVES];
+  return wsum[wave] + inc - v;
+}
+
+__global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
+    int32_t *__restrict__ plan, const int64_t *__restrict__ ids, const int64_t *__restrict__ a_start,
+    const int64_t *__restrict__ a_len, int T, int A, int n_slots, int bm_s, int bm_e, int W,
+    int64_t off_perm, int64_t off_padapter, int64_t off_prank, int64_t off_tiles_s,
+    int64_t off_tiles_e, int64_t off_scratch) {
+  __shared__ int32_t whist[HIST_WORDS];
+  __shared__ int wsum[PLAN_WAVES + 1];
+  __shared__ int s_maxrank;
+  __shared__ int s_err;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int32_t *perm = plan + off_perm;
+  int32_t *padapter = plan + off_padapter;
+  int32_t *prank = plan + off_prank;
+  int32_t *cnt = plan + off_scratch;
+  int32_t *gstart = cnt + A;
+  int32_t *toff_s = gstart + A;
+  int32_t *toff_e = toff_s + A;
+
+  for (int i = tid; i < W * A; i += PLAN_THREADS) whist[i] = 0;
+  if (tid == 0) { s_maxrank = 0; s_err = 0; }
+  __syncthreads();
+
+  // token range of each of the W histogram waves (contiguous, multiple of 64)
+  const int cw = (int)align_up((T + W - 1) / W, 64);
+  const int t_beg = wave * cw;
+  const int t_end = (wave < W) ? min(T, t_beg + cw) : 0;
+
+  // 1. per-wave histogram of valid tokens
+  for (int t = t_beg + lane; t < t_end; t += 64) {
+    const int64_t a = ids[t];
+    if (a >= 0 && a < A && (a_len[a] / n_slots) > 0) atomicAdd(&whist[wave * A + (int)a], 1);
+  }
+  __syncthreads();
+
+  // 2. per-adapter totals, group starts, tile offsets (each thread owns a run of adapters)
+  const int per = (A + PLAN_THREADS - 1) / PLAN_THREADS;
+  const int a_beg = min(A, tid * per), a_endx = min(A, a_beg + per);
+  int my_c = 0, my_ts = 0, my_te = 0, my_g = 0, my_maxr = 0;
+  for (int a = a_beg; a < a_endx; ++a) {
+    int c = 0;
+    for (int w = 0; w < W; ++w) c += whist[w * A + a];
+    cnt[a] = c;
+    if (c > 0) {
+      my_c += c;
+      my_ts += (c + bm_s - 1) / bm_s;
+      my_te += (c + bm_e - 1) / bm_e;
+      my_g += 1;
+      my_maxr = max(my_maxr, (int)(a_len[a] / n_slots));
+    }
+  }
+  int n_active, n_ts, n_te, n_g;
+  int pre_c = block_exclusive_scan(my_c, &n_active, wsum);
+  int pre_ts = block_exclusive_scan(my_ts, &n_ts, wsum);
+  int pre_te = block_exclusive_scan(my_te, &n_te, wsum);
+  (void)block_exclusive_scan(my_g, &n_g, wsum);
+  if (my_maxr > 0) atomicMax(&s_maxrank, my_maxr);
+  for (int a = a_beg; a < a_endx; ++a) {
+    const int c = cnt[a];
+    gstart[a] = pre_c;
+    toff_s[a] = pre_ts;
+    toff_e[a] = pre_te;
+    int off = pre_c;
+    for (int w = 0; w < W; ++w) {  // histogram -> running write offset of (wave, adapter)
+      const int h = whist[w * A + a];
+      whist[w * A + a] = off;
+      off += h;
+    }
+    pre_c += c;
+    pre_ts += (c + bm_s - 1) / bm_s;
+    pre_te += (c + bm_e - 1) / bm_e;
+  }
+  __syncthreads();
+
+  // 3. stable scatter: each wave walks its range in order, 64 tokens a step; lanes holding the
+  //    same adapter get consecutive positions in lane order.
+  for (int t0 = t_beg; t0 < t_end; t0 += 64) {
+    const int t = t0 + lane;
+    int a = -1, r = 0;
+    if (t < t_end) {
+      const int64_t a64 = ids[t];
+      if (a64 >= 0 && a64 < A) {
+        r = (int)(a_len[a64] / n_slots);
+        if (r > 0) a = (int)a64;
+      }
+    }
+    unsigned long long remaining = __ballot(a >= 0);
+    while (remaining) {
+      const int leader = __ffsll((long long)remaining) - 1;
+      const int a0 = __shfl(a, leader, 64);
+      const unsigned long long m = __ballot(a == a0);
+      const int slot_idx = wave * A + a0;
+      const int base = whist[slot_idx];
+      if (a == a0) {
+        const int pos = base + __popcll(m & ((1ull << lane) - 1ull));
+        perm[pos] = t;
+        padapter[pos] = a0;
+        prank[pos] = r;
+      }
+      __builtin_amdgcn_wave_barrier();
+      if (lane == leader) whist[slot_idx] = base + __popcll(m);
+      __builtin_amdgcn_wave_barrier();
+      remaining &= ~m;
+    }
+  }
+  __syncthreads();
+
+  // 4. tile lists: tile i belongs to the last adapter whose tile offset is <= i
+  for (int pass = 0; pass < 2; ++pass) {
+    const int n_tiles = pass ? n_te : n_ts;
+    const int bm = pass ? bm_e : bm_s;
+    const int32_t *toff = pass ? toff_e : toff_s;
+    int32_t *tiles = plan + (pass ? off_tiles_e : off_tiles_s);
+    for (int i = tid; i < n_tiles; i += PLAN_THREADS) {
+      int lo = 0, hi = A;  // first adapter with toff > i
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (toff[mid] <= i) lo = mid + 1; else hi = mid;
+      }
+      const int a = lo - 1;
+      const int k = i - toff[a];
+      const int c = cnt[a];
+      const int64_t st = a_start[a];
+      if (st < 0 || st > 0x7fffffff) atomicOr(&s_err, (int)PERR_START_OVERFLOW);
+      int32_t *tl = tiles + (int64_t)i * TILE_WORDS;
+      tl[0] = a;
+      tl[1] = (int)(a_len[a] / n_slots);
+      tl[2] = gstart[a] + k * bm;
+      tl[3] = min(bm, c - k * bm);
+      tl[4] = (int32_t)st;
+      tl[5] = 0; tl[6] = 0; tl[7] = 0;
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    plan[H_MAGIC] = PLAN_MAGIC;
+    plan[H_T] = T;
+    plan[H_NADAPTERS] = A;
+    plan[H_NTILES_S] = n_ts;
+    plan[H_NTILES_E] = n_te;
+    plan[H_NGROUPS] = n_g;
+    plan[H_MAXRANK] = s_maxrank;
+    plan[H_ERR] = s_err;
+    plan[H_BM_S] = bm_s;
+    plan[H_BM_E] = bm_e;
+    plan[H_NACTIVE] = n_active;
+  }
+}
+
+// Parallel RLE.  Pass 1 marks run heads and scans them; pass 2 derives the run lengths.
+__global__ __launch_bounds__(PLAN_THREADS) void count_consecutive_kernel(
+    const int64_t *__restrict__ lora_rank, int64_t n_adapters, const int64_t *__restrict__ indicies,
+    int T, int64_t *__restrict__ output_counts, int64_t *__restrict__ rank_counts,
+    int64_t *__restrict__ lora_ids, int64_t *__restrict__ start_ids, int64_t *__restrict__ num_runs) {
+  __shared__ int wsum[PLAN_WAVES + 1];
+  const int tid = threadIdx.x;
+  int carry = 0;
+  for (int t0 = 0; t0 < T; t0 += PLAN_THREADS) {
+    const int t = t0 + tid;
+    int head = 0;
+    int64_t id = 0;
+    if (t < T) {
+      id = indicies[t];
+      head = (t == 0) || (indicies[t - 1] != id);
+    }
+    int total;
+    const int pre = block_exclusive_scan(head, &total, wsum);
+    if (head) {
+      const int k = carry + pre;
+      start_ids[k] = t;
+      lora_ids[k] = id;
+      rank_counts[k] = (id >= 0 && id < n_adapters) ? lora_rank[id] / 4 : 0;
+    }
+    carry += total;
+  }
+  __syncthreads();  // start_ids written by this workgroup are visible to it
+  const int P = carry;
+  for (int k = tid; k < P; k += PLAN_THREADS) {
+    const int64_t s = start_ids[k];
+    const int64_t e = (k + 1 < P) ? start_ids[k + 1] : (int64_t)T;
+    output_counts[k] = e - s;
+  }
+  if (tid == 0) num_runs[0] = P;
+}
+
+__global__ void ids_fill_kernel(int64_t *ids_out, int64_t T, int64_t v) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < T) ids_out[t] = v;
+}
+
+__global__ void ids_cover_segments_kernel(int64_t *ids_out, const int64_t *ids_in,
+                                          const int64_t *start_ids, const int64_t *output_counts,
+                                          int64_t T) {
+  const int64_t i = blockIdx.x;
+  const int64_t s = start_ids[i], n = output_counts[i];
+  if (s < 0 || n <= 0) return;
+  const int64_t e = (s + n < T) ? s + n : T;
+  for (int64_t t = s + threadIdx.x; t < e; t += blockDim.x) ids_out[t] = ids_in[t];
+}
+
+__global__ void ids_cover_requests_kernel(int64_t *ids_out, const int32_t *b_start_loc,
+                                          const int32_t *b_seq_len, const int64_t *b_indicies,
+                                          int64_t T, int64_t max_rows) {
+  const int64_t i = blockIdx.x;
+  const int64_t s = b_start_loc[i];
+  int64_t n = b_seq_len[i];
+  if (n > max_rows) n = max_rows;
+  if (s < 0 || n <= 0) return;
+  const int64_t e = (s + n < T) ? s + n : T;
+  const int64_t a = b_indicies[i];
+  for (int64_t t = s + threadIdx.x; t < e; t += blockDim.x) ids_out[t] = a;
+}
+
+}  // namespace
+
+int launch_plan(hipStream_t st, int32_t *plan, const PlanLayout &L, const int64_t *ids,
+                const int64_t *a_start, const int64_t *a_len, int n_slots, int bm_s, int bm_e) {
+  const int A = (int)L.A;
+  int W = A > 0 ? (int)(HIST_WORDS / A) : PLAN_WAVES;
+  if (W > PLAN_WAVES) W = PLAN_WAVES;
+  if (W < 1) return fail(MLORA_ERR_NO_KERNEL, "plan: more than %lld adapters", (long long)MAX_ADAPTERS);
+  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(PLAN_THREADS), 0, st, plan, ids, a_start, a_len,
+                     (int)L.T, A, n_slots, bm_s, bm_e, W, L.off_perm, L.off_padapter, L.off_prank,
+                     L.off_tiles_s, L.off_tiles_e, L.off_scratch);
+  return check_launch("plan_kernel");
+}
+
+int launch_count_consecutive(hipStream_t st, const int64_t *lora_rank, int64_t n_adapters,
+                             const int64_t *indicies, int64_t T, int64_t *output_counts,
+                             int64_t *rank_counts, int64_t *lora_ids, int64_t *start_ids,
+                             int64_t *num_runs) {
+  hipLaunchKernelGGL(count_consecutive_kernel, dim3(1), dim3(PLAN_THREADS), 0, st, lora_rank,
+                     n_adapters, indicies, (int)T, output_counts, rank_counts, lora_ids, start_ids,
+                     num_runs);
+  return check_launch("count_consecutive_kernel");
+}
+
+int launch_ids_from_segments(hipStream_t st, int64_t *ids_out, const int64_t *ids_in,
+                             const int64_t *start_ids, const int64_t *output_counts, int64_t P,
+                             int64_t T) {
+  if (T <= 0) return MLORA_OK;
+  hipLaunchKernelGGL(ids_fill_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, ids_out, T,
+                     (int64_t)-1);
+  if (int rc = check_launch("ids_fill_kernel")) return rc;
+  if (P <= 0) return MLORA_OK;
+  hipLaunchKernelGGL(ids_cover_segments_kernel, dim3((unsigned)P), dim3(256), 0, st, ids_out, ids_in,
+                     start_ids, output_counts, T);
+  return check_launch("ids_cover_segments_kernel");
+}
+
+int launch_ids_from_requests(hipStream_t st, int64_t *ids_out, const int32_t *b_start_loc,
+                             const int32_t *b_seq_len, const int64_t *b_indicies, int64_t n_req,
+                             int64_t T, int64_t max_rows) {
+  if (T <= 0) return MLORA_OK;
+  hipLaunchKernelGGL(ids_fill_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st, ids_out, T,
+                     (int64_t)-1);
+  if (int rc = check_launch("ids_fill_kernel")) return rc;
+  if (n_req <= 0) return MLORA_OK;
+  hipLaunchKernelGGL(ids_cover_requests_kernel, dim3((unsigned)n_req), dim3(256), 0, st, ids_out,
+                     b_start_loc, b_seq_len, b_indicies, T, max_rows);
+  return check_launch("ids_cover_requests_kernel");
+}
+
+}  // namespace mlora

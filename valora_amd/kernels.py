@@ -1,0 +1,73 @@
+"""Drop-in for the reference's BGMV extension ``valora._kernels``.
+
+``dispatch_bgmv`` keeps the reference's positional signature, argument meaning, in-place
+behaviour and error behaviour (valora/csrc/lora_ops.cc:76-126); the work is done by the gfx950
+kernels behind ``libmlora.so``.  Call sites it serves:
+valora/models/peft/lora_unordered_batch_infer.py:632-638,1141-1148,1521-1527.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def _check_input(t: torch.Tensor, name: str) -> None:
+    # CHECK_INPUT = CHECK_CUDA + CHECK_CONTIGUOUS (valora/csrc/lora_ops.cc:27-34)
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def _check_common(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies):
+    for t, n in ((y, "y"), (x, "x"), (w, "w"), (start_indicies, "start_indicies"),
+                 (lora_ranks, "lora_ranks"), (loc_indicies, "loc_indicies"), (indicies, "indicies")):
+        _check_input(t, n)
+    if y.dim() != 2:
+        raise RuntimeError("y must be a 2D tensor")
+    if x.dim() != 2:
+        raise RuntimeError("x must be a 2D tensor")
+    if w.dim() != 3:
+        raise RuntimeError("w must be a 3D tensor")
+    if indicies.dim() != 1:
+        raise RuntimeError("indicies must be a 1D tensor")
+    if indicies.size(0) != x.size(0):
+        raise RuntimeError(f"CHECK_EQ(indicies.size(0), x.size(0)) failed. {indicies.size(0)} vs {x.size(0)}")
+    if y.size(0) != x.size(0):
+        raise RuntimeError(f"CHECK_EQ(y.size(0), x.size(0)) failed. {y.size(0)} vs {x.size(0)}")
+    for t, n in ((start_indicies, "start_indicies"), (lora_ranks, "lora_ranks"),
+                 (loc_indicies, "loc_indicies"), (indicies, "indicies")):
+        if t.dtype != torch.long:  # data_ptr<int64_t>() throws on any other type
+            raise RuntimeError(f"expected scalar type Long but found {t.dtype} ({n})")
+
+
+def _no_kernel(h_in, h_out, dtype):
+    return RuntimeError(f"No suitable kernel. h_in={h_in} h_out={h_out} dtype={dtype}")
+
+
+def _workspace(T: int, n_adapters: int, narrow: int, device) -> torch.Tensor:
+    n = _lib.lib().mlora_workspace_bytes(T, n_adapters, narrow)
+    return torch.empty(max(int(n), 256), dtype=torch.uint8, device=device)
+
+
+def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales) -> None:
+    """In place on ``y``.  ``h_in > h_out``: shrink ``y[t, :r] = x[t] @ A_a.T`` (columns >= r keep
+    their value); ``h_in < h_out``: expand ``y[t] += scale_a * x[t, :r] @ B_a``.  ``lora_ranks``
+    holds ``4 * r``; ``w`` is the pool ``[rows, heads, head_dim]`` whose row width is the wide
+    dimension of the call."""
+    _check_common(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies)
+    T, h_in, h_out = x.size(0), x.size(1), y.size(1)
+    code = _lib.dtype_code(x.dtype)
+    if code < 0 or y.dtype != x.dtype or w.dtype != x.dtype:
+        raise _no_kernel(h_in, h_out, x.dtype)
+    if not (h_in < 65536 and h_out < 65536):
+        raise _no_kernel(h_in, h_out, x.dtype)
+    wide = max(h_in, h_out)
+    if lora_scales is not None and lora_scales.dtype != x.dtype:
+        lora_scales = lora_scales.to(x.dtype)  # the kernel reads scales as T (bgmv_impl.cuh:180)
+    pool = _lib.make_pool(w, start_indicies, lora_ranks, loc_indicies, wide, 4)
+    ws = _workspace(T, start_indicies.numel(), min(h_in, h_out), x.device)
+    _lib.check(_lib.lib().mlora_dispatch_bgmv(
+        _lib.current_stream(x.device), _lib.ptr(y), _lib.ptr(x), pool, _lib.ptr(indicies), int(qkvo),
+        _lib.ptr(lora_scales), T, h_in, h_out, code, _lib.ptr(ws), ws.numel()))

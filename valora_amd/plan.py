@@ -1,0 +1,108 @@
+"""Planned multi-LoRA op: build the adapter-grouped work tiles once per batch, then apply
+shrink + expand for every (layer, target) of the step.
+
+The reference rebuilds its segment tensors once per forward
+(valora/server/router/model_infer/model_rpc.py:381) and then issues 8 op launches per layer with
+the same per-token ids (valora/models/peft/lora_unordered_batch_infer.py:946-988,1611-1622);
+``LoraPlan`` is that once-per-forward object for the gfx950 kernels.  The intermediate
+``v = x @ A.T`` never becomes a caller-visible tensor: it lives in an fp32 split-K buffer between
+the two launches and is rounded to the operand dtype exactly once, where the reference stores
+its ``delta`` tensor.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib, tile_table
+
+
+class LoraPlan:
+    def __init__(self, ids: torch.Tensor, a_start: torch.Tensor, a_len: torch.Tensor, max_rank: int,
+                 n_slots: int = 4, hidden: int = 4096, bm_shrink: Optional[int] = None,
+                 bm_expand: Optional[int] = None, ksplit: Optional[int] = None):
+        """``ids``: int64 per-token adapter index (negative = no adapter); ``a_start`` / ``a_len``:
+        the pool index (``a_len = n_slots * rank``); ``max_rank``: widest rank among the resident
+        adapters (the reference's ``max_lora_dim``, lora_unordered_batch_infer.py:181-182)."""
+        if not ids.is_cuda:
+            raise RuntimeError("ids must be a CUDA tensor")
+        if ids.dtype != torch.long or a_start.dtype != torch.long or a_len.dtype != torch.long:
+            raise RuntimeError("expected scalar type Long")
+        self.device = ids.device
+        self.T = int(ids.numel())
+        self.n_adapters = int(a_start.numel())
+        self.n_slots = n_slots
+        self.max_rank = int(max_rank)
+        cfg = tile_table.lookup(self.T, self.max_rank, hidden, self.n_adapters)
+        self.bm_shrink = cfg.bm_shrink if bm_shrink is None else bm_shrink
+        self.bm_expand = cfg.bm_expand if bm_expand is None else bm_expand
+        self.ksplit = cfg.ksplit if ksplit is None else ksplit
+        L = _lib.lib()
+        nbytes = int(L.mlora_plan_bytes(self.T, self.n_adapters))
+        self.buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
+        self.handle = _lib.Plan(_lib.ptr(self.buf), self.buf.numel(), 0, 0, 0, 0)
+        self._keep = (ids, a_start, a_len)
+        _lib.check(L.mlora_build_plan(_lib.current_stream(self.device), self.handle, _lib.ptr(ids.contiguous()),
+                                      self.T, _lib.ptr(a_start), _lib.ptr(a_len), self.n_adapters, n_slots,
+                                      self.bm_shrink, self.bm_expand))
+        pbytes = int(L.mlora_partial_bytes(self.T, self.max_rank, max(self.ksplit, 1)))
+        self.partial = torch.empty(pbytes // 4, dtype=torch.float32, device=self.device)
+
+    # -- introspection (synchronises; for tests and diagnostics) --------------------------------
+    def header(self) -> dict:
+        h = self.buf[:128].view(torch.int32).cpu().tolist()
+        names = ["magic", "T", "n_adapters", "n_tiles_shrink", "n_tiles_expand", "n_groups", "max_rank",
+                 "err", "bm_shrink", "bm_expand", "n_active"]
+        return dict(zip(names, h))
+
+    def perm(self) -> torch.Tensor:
+        n = self.header()["n_active"]
+        return self.buf.view(torch.int32)[32:32 + n].clone()
+
+    def _section(self, index: int) -> torch.Tensor:
+        # layout mirrors plan_layout() in csrc/mlora_internal.h
+        T, A = self.T, self.n_adapters
+        up8 = lambda v: (v + 7) // 8 * 8
+        max_tiles = (T + 15) // 16 + min(A, T)
+        off_perm = 32
+        off_pad = up8(off_perm + T)
+        off_prank = up8(off_pad + T)
+        off_ts = up8(off_prank + T)
+        off_te = off_ts + max_tiles * 8
+        words = self.buf.view(torch.int32)
+        h = self.header()
+        if index == 0:
+            return words[off_pad:off_pad + h["n_active"]].clone()
+        if index == 1:
+            return words[off_prank:off_prank + h["n_active"]].clone()
+        if index == 2:
+            return words[off_ts:off_ts + h["n_tiles_shrink"] * 8].view(-1, 8).clone()
+        return words[off_te:off_te + h["n_tiles_expand"] * 8].view(-1, 8).clone()
+
+    def position_adapters(self): return self._section(0)
+    def position_ranks(self): return self._section(1)
+    def tiles_shrink(self): return self._section(2)
+    def tiles_expand(self): return self._section(3)
+
+    # -- the op -------------------------------------------------------------------------------------
+    def apply(self, y: torch.Tensor, x: torch.Tensor, key_buffer: torch.Tensor, value_buffer: torch.Tensor,
+              a_start: torch.Tensor, a_len: torch.Tensor, a_loc: torch.Tensor, slot: int,
+              scales: torch.Tensor) -> None:
+        """``y[t] += scale_a * (x[t] @ A_a.T) @ B_a`` in place for every token with an adapter."""
+        if x.dim() != 2 or y.dim() != 2 or x.size(0) != self.T or y.size(0) != self.T:
+            raise RuntimeError(f"x and y must be [T={self.T}, H] matrices")
+        if not (x.is_contiguous() and y.is_contiguous()):
+            raise RuntimeError("x and y must be contiguous")
+        code = _lib.dtype_code(x.dtype)
+        if code < 0 or y.dtype != x.dtype or key_buffer.dtype != x.dtype or value_buffer.dtype != x.dtype:
+            raise RuntimeError(f"No suitable kernel. h_in={x.size(1)} h_out={y.size(1)} dtype={x.dtype}")
+        if scales.dtype != x.dtype:
+            scales = scales.to(x.dtype)
+        h_in, h_out = x.size(1), y.size(1)
+        pa = _lib.make_pool(key_buffer, a_start, a_len, a_loc, h_in, self.n_slots)
+        pb = _lib.make_pool(value_buffer, a_start, a_len, a_loc, h_out, self.n_slots)
+        _lib.check(_lib.lib().mlora_lora_apply(
+            _lib.current_stream(self.device), self.handle, _lib.ptr(self.partial), self.partial.numel() * 4,
+            _lib.ptr(y), _lib.ptr(x), self.T, h_in, h_out, self.max_rank, pa, pb, int(slot), _lib.ptr(scales),
+            int(self.ksplit), code))

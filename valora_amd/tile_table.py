@@ -1,0 +1,76 @@
+"""Tile-configuration table for the gfx950 LoRA kernels.
+
+Replaces the reference's ``shape_to_config`` dictionary and ``get_config_a`` / ``get_config_b``
+(valora/models/peft/lora_unordered_batch_infer.py:25-172,216-236), which map
+``(n_adapters, first_seq_len, K, N)`` to CUTLASS threadblock / warp shapes tuned on an A100 and
+fall back to a fixed shape for unknown keys.  Here the key is
+``(token bucket, max rank, hidden, adapter bucket)`` and the value is what the HIP kernels can
+vary: the token height of a shrink tile, the split-K factor of the shrink and the token height
+of an expand tile.  Entries come from sweeps on MI355X (``tile_table.json`` next to this file);
+unknown keys fall back to a rule, like the reference's fallback tuple.
+"""
+from __future__ import annotations
+
+import json
+import os
+from dataclasses import dataclass
+from typing import Dict, Tuple
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+TABLE_PATH = os.path.join(_HERE, "tile_table.json")
+
+TOKEN_BUCKETS = (64, 256, 1024, 4096, 16384, 1 << 22)
+ADAPTER_BUCKETS = (1, 8, 32, 128, 8192)
+
+
+@dataclass(frozen=True)
+class TileConfig:
+    bm_shrink: int   # tokens per shrink tile: 16, 32 or 64
+    ksplit: int      # K-chunks the shrink is split into (partials summed by the consumer)
+    bm_expand: int   # tokens per expand tile: multiple of 16 up to 256
+
+
+def _bucket(v: int, buckets) -> int:
+    for b in buckets:
+        if v <= b:
+            return b
+    return buckets[-1]
+
+
+def key(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> str:
+    return f"{_bucket(n_tokens, TOKEN_BUCKETS)}:{max_rank}:{hidden}:{_bucket(n_adapters, ADAPTER_BUCKETS)}"
+
+
+def fallback(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> TileConfig:
+    bm_s = 16 if n_tokens <= 2048 else 32 if n_tokens <= 8192 else 64
+    if max_rank > 64:
+        bm_s = min(bm_s, 32)
+    tiles = max(1, min(n_tokens, -(-n_tokens // bm_s) + min(n_adapters, n_tokens)))
+    ksplit = max(1, min(16, hidden // 256, -(-1024 // tiles)))
+    bm_e = 32 if n_tokens <= 1024 else 64 if n_tokens <= 8192 else 128
+    return TileConfig(bm_s, ksplit, bm_e)
+
+
+_table: Dict[str, TileConfig] = {}
+_loaded = False
+
+
+def _load() -> None:
+    global _loaded
+    _loaded = True
+    if os.path.exists(TABLE_PATH):
+        with open(TABLE_PATH) as f:
+            raw = json.load(f)
+        for k, v in raw.get("entries", {}).items():
+            _table[k] = TileConfig(int(v["bm_shrink"]), int(v["ksplit"]), int(v["bm_expand"]))
+
+
+def lookup(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> TileConfig:
+    if not _loaded:
+        _load()
+    cfg = _table.get(key(n_tokens, max_rank, hidden, n_adapters))
+    if cfg is None:
+        return fallback(n_tokens, max_rank, hidden, n_adapters)
+    if max_rank > 64 and cfg.bm_shrink > 32:
+        cfg = TileConfig(32, cfg.ksplit, cfg.bm_expand)
+    return cfg
