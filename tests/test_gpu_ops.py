@@ -14,7 +14,8 @@ pytestmark = pytest.mark.gpu
 
 def _case(seed, T, h_in, h_out, ranks, dtype, paged=True, id_style="random", scal=None):
     g = torch.Generator().manual_seed(seed)
-    pool = W.make_pool(list(ranks), h_in, h_out, dtype, g, paged, std=0.05, scalings=scal)
+    heads = 32 if h_in % 32 == 0 and h_out % 32 == 0 else 8
+    pool = W.make_pool(list(ranks), h_in, h_out, dtype, g, paged, std=0.05, scalings=scal, heads=heads)
     A = len(ranks)
     if id_style == "random":
         ids = torch.randint(0, A, (T,), generator=g)

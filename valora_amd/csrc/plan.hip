@@ -78,7 +78,10 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
   // 1. per-wave histogram of valid tokens
   for (int t = t_beg + lane; t < t_end; t += 64) {
     const int64_t a = ids[t];
-    if (a >= 0 && a < A && (a_len[a] / n_slots) > 0) atomicAdd(&whist[wave * A + (int)a], 1);
+    if (a >= 0 && a < A) {
+      const int64_t r = a_len[a] / n_slots;   // ranks are multiples of 8 (16-byte vectors)
+      if (r > 0 && (r & 7) == 0 && r <= MAX_RANK) atomicAdd(&whist[wave * A + (int)a], 1);
+    }
   }
   __syncthreads();
 
@@ -130,7 +133,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
       const int64_t a64 = ids[t];
       if (a64 >= 0 && a64 < A) {
         r = (int)(a_len[a64] / n_slots);
-        if (r > 0) a = (int)a64;
+        if (r > 0 && (r & 7) == 0 && r <= MAX_RANK) a = (int)a64;
       }
     }
     unsigned long long remaining = __ballot(a >= 0);

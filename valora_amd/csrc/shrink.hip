@@ -67,12 +67,16 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs p) {
 
   const int kbeg = s * p.kchunk;
   const int kend = min(p.h_in, kbeg + p.kchunk);
-  for (int k = kbeg + wave * 32 + kg * 8; k < kend; k += 128) {
+  // The trip count must be wave-uniform: MFMA ignores EXEC, so a lane that left the loop early
+  // would still feed its stale registers into the matrix core.  Lanes past the end load zeros.
+  for (int kb = kbeg + wave * 32; kb < kend; kb += 128) {
+    const int k = kb + kg * 8;
+    const bool kok = k < kend;
     u32x4 xa[MB], wb[NB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) xa[mb] = xok[mb] ? load16(xp[mb] + k) : u32x4{0, 0, 0, 0};
+    for (int mb = 0; mb < MB; ++mb) xa[mb] = (xok[mb] && kok) ? load16(xp[mb] + k) : u32x4{0, 0, 0, 0};
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) wb[nb] = wok[nb] ? load16(wp[nb] + k) : u32x4{0, 0, 0, 0};
+    for (int nb = 0; nb < NB; ++nb) wb[nb] = (wok[nb] && kok) ? load16(wp[nb] + k) : u32x4{0, 0, 0, 0};
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
       if (nb * 16 < r) {
