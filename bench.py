@@ -1,0 +1,287 @@
+#!/usr/bin/env python3
+"""Benchmark of the multi-LoRA batching operator on one MI355X.
+
+Workload (the shape the headline metric is quoted on): decode BGMV -- 256 tokens, one per
+request, x[256,4096] fp16, 64 resident adapters of rank 16, per-token adapter id ~ Zipf(0.6),
+4096 -> 4096, y += scale * (x @ A_a.T) @ B_a.  One *step* is one decode step's worth of this op:
+the op applied on `--layers` (32) different layers, each with its own pool slice, x and y, so the
+operands of consecutive launches do not sit in cache.  The layer loop is captured in a HIP graph
+(the op allocates nothing and only launches kernels on the caller's stream) and replayed.
+
+Prints ONE JSON line: value = microseconds per LoRA layer-op; `roofline` = achieved algorithmic
+HBM bytes/s of the dominant kernel against the 8 TB/s peak, measured with HIP events on the launch
+stream; `cpu_baseline` = the reference's PyTorch per-segment path restated on CPU, timed on this
+host's cores on the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
+# scaled by the same counters' reading for a plain copy of known size; None until measured.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly from Python instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--bm-shrink", type=int, default=None)
+    ap.add_argument("--bm-expand", type=int, default=None)
+    ap.add_argument("--ksplit", type=int, default=None)
+    ap.add_argument("--all-configs", metavar="FILE", default=None,
+                    help="also measure every target of configs 1,3,4,5 and write a JSON report to FILE")
+    return ap.parse_args()
+
+
+def build_layers(torch, W, dev, L):
+    """Layer 0 is the seeded benchmark workload; the other layers reuse its ids and pool index
+    (the reference shares a_start/a_len/a_loc across layers and indexes key_buffer[layer]) with
+    their own random weights, x and y."""
+    w = W.config2()
+    wd = w.to(dev)
+    t = wd.targets[0]
+    p = t.pool
+    g = torch.Generator(device=dev).manual_seed(2002)
+    kb, vb, xs, ys = [p.key_buffer], [p.value_buffer], [wd.x[4096]], [wd.y0["q"].clone()]
+    for _ in range(1, L):
+        kb.append((torch.randn(p.key_buffer.shape, generator=g, device=dev) * 0.02).to(w.dtype))
+        vb.append((torch.randn(p.value_buffer.shape, generator=g, device=dev) * 0.02).to(w.dtype))
+        xs.append(torch.randn(w.T, 4096, generator=g, device=dev).to(w.dtype))
+        ys.append(torch.randn(w.T, 4096, generator=g, device=dev).to(w.dtype))
+    return w, wd, kb, vb, xs, ys
+
+
+def time_graph(torch, fn, reps, warm, use_graph):
+    """Average milliseconds of one call of fn() (which enqueues work on the current stream),
+    from HIP events recorded on that stream around `reps` back-to-back repetitions."""
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(2):
+            fn()
+        graph = None
+        if use_graph:
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=s):
+                fn()
+        run = graph.replay if graph is not None else fn
+        for _ in range(warm):
+            run()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(reps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / reps
+        ev_ms = e0.elapsed_time(e1) / reps
+    torch.cuda.current_stream().wait_stream(s)
+    return ev_ms, wall_ms
+
+
+def cpu_baseline(torch, w, budget_s=15.0):
+    """The reference's per-segment PyTorch path (valora/models/bmm/lora_bmm_infer.py:342-352)
+    restated in oracle/, on this host's cores: decode tokens are length-1 segments after grouping
+    consecutive equal ids."""
+    from oracle import lora_oracle as O
+    t = w.targets[0]
+    p = t.pool
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    dense = [p.dense(a, t.slot) for a in range(p.n_adapters)]
+    A_list, B_list = [d[0] for d in dense], [d[1] for d in dense]
+    segs = O.segments_from_ids(w.ids.tolist())
+    scal = [float(s) for s in p.a_scaling]
+    x, y0 = w.x[t.h_in], w.y0[t.name]
+    kind = "native " + str(w.dtype).replace("torch.", "")
+    compute = None
+    try:
+        t0 = time.perf_counter()
+        O.per_segment_mm(y0, x, A_list, B_list, segs, scal)
+        first = time.perf_counter() - t0
+        if first > 2.0:
+            raise RuntimeError("16-bit CPU matmul too slow")
+    except Exception:
+        compute, kind = torch.float32, "fp32 compute on 16-bit-rounded inputs"
+    for _ in range(3):
+        O.per_segment_mm(y0, x, A_list, B_list, segs, scal, compute_dtype=compute)
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 10 or (time.perf_counter() - t_start < budget_s and len(times) < 2000):
+        t0 = time.perf_counter()
+        O.per_segment_mm(y0, x, A_list, B_list, segs, scal, compute_dtype=compute)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": round(med * 1e6, 2), "unit": "us/layer", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{len(times)} repetitions of the full config-2 op (256 tokens -> {len(segs)} segments), "
+                      f"median; {kind}; min {times[0] * 1e6:.1f} us"}
+
+
+def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph):
+    """Per-target timing of the other benchmark configurations (report only; the JSON line of the
+    default run is config 2).  Each target's shrink+expand is replayed back to back on `reps`
+    copies of y so that the read-modify-write does not hit the same lines."""
+    report = {}
+    for n in (1, 3, 4, 5):
+        w = W.CONFIGS[n]()
+        wd = w.to(dev)
+        R = max(w.targets[0].pool.ranks)
+        rows = {}
+        total_us = 0.0
+        for t in wd.targets:
+            p = t.pool
+            plan = LoraPlan(wd.ids, p.a_start, p.a_len, R, hidden=t.h_in)
+            ycopies = [wd.y0[t.name].clone() for _ in range(4)]
+            x = wd.x[t.h_in]
+
+            def fn():
+                for yy in ycopies:
+                    plan.apply(yy, x, p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
+
+            def fs():
+                for yy in ycopies:
+                    plan.shrink(x, p.key_buffer, p.a_start, p.a_len, p.a_loc, t.slot)
+
+            def fe():
+                for yy in ycopies:
+                    plan.expand(yy, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
+
+            ms, _ = time_graph(torch, fn, 30, 3, use_graph)
+            ms_s, _ = time_graph(torch, fs, 30, 3, use_graph)
+            ms_e, _ = time_graph(torch, fe, 30, 3, use_graph)
+            us = ms * 1e3 / 4
+            b, f = w.algorithmic_bytes(t.name), w.flops(t.name)
+            rows[t.name] = {"us": round(us, 2), "shrink_us": round(ms_s * 250, 2), "expand_us": round(ms_e * 250, 2),
+                            "bytes": b, "flops": f, "gbps": round(b / us / 1e3, 1),
+                            "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4), "tflops": round(f / us / 1e6, 2),
+                            "tile": [plan.bm_shrink, plan.ksplit, plan.bm_expand]}
+            total_us += us
+        report[f"config{n}"] = {"tokens": w.T, "dtype": str(w.dtype), "max_rank": R, "targets": rows,
+                                "us_per_layer": round(total_us, 2)}
+        del wd
+        torch.cuda.empty_cache()
+    with open(path, "w") as f:
+        json.dump(report, f, indent=1)
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (nothing in this build uses a second GPU)",
+              file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from valora_amd import workloads as W
+    from valora_amd.plan import LoraPlan
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    L = args.layers
+    w, wd, kb, vb, xs, ys = build_layers(torch, W, dev, L)
+    t = wd.targets[0]
+    p = t.pool
+    plan = LoraPlan(wd.ids, p.a_start, p.a_len, 16, hidden=4096, bm_shrink=args.bm_shrink,
+                    bm_expand=args.bm_expand, ksplit=args.ksplit)
+    idx = (p.a_start, p.a_len, p.a_loc)
+    use_graph = not args.no_graph
+
+    def step():
+        for l in range(L):
+            plan.apply(ys[l], xs[l], kb[l], vb[l], *idx, 0, p.a_scaling)
+
+    def shrink_only():
+        for l in range(L):
+            plan.shrink(xs[l], kb[l], *idx, 0)
+
+    def expand_only():
+        for l in range(L):
+            plan.expand(ys[l], vb[l], *idx, 0, p.a_scaling)
+
+    # ---- the timed region: W warm-up steps, then exactly K steps between two synchronisations
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        step()
+        graph = None
+        if use_graph:
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=s):
+                step()
+        run = graph.replay if graph is not None else step
+        for _ in range(args.warmup):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            run()
+        torch.cuda.synchronize()
+        ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    torch.cuda.current_stream().wait_stream(s)
+    us_per_layer = ms_per_step * 1e3 / L
+
+    # ---- per-kernel durations (HIP events on the launch stream, same layer rotation)
+    reps = max(10, min(args.steps, 200))
+    sh_ms, _ = time_graph(torch, shrink_only, reps, 5, use_graph)
+    ex_ms, _ = time_graph(torch, expand_only, reps, 5, use_graph)
+    op_ms, _ = time_graph(torch, step, reps, 5, use_graph)
+    sh_us, ex_us, op_us = sh_ms * 1e3 / L, ex_ms * 1e3 / L, op_ms * 1e3 / L
+
+    s_el = 2
+    used = sorted(set(w.ids.tolist()))
+    r_sum = sum(w.targets[0].pool.ranks[a] for a in used)
+    bytes_shrink = w.T * 4096 * s_el + r_sum * 4096 * s_el
+    bytes_expand = r_sum * 4096 * s_el + 2 * w.T * 4096 * s_el
+    bytes_op = w.algorithmic_bytes("q")
+    assert bytes_op == bytes_shrink + bytes_expand
+    dom = ("expand_kernel", bytes_expand, ex_us) if ex_us >= sh_us else ("shrink_kernel", bytes_shrink, sh_us)
+    achieved = dom[1] / (dom[2] * 1e-6) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                "kernel": dom[0], "algorithmic_bytes_per_launch": dom[1], "avg_launch_us": round(dom[2], 3),
+                "shrink_kernel_us": round(sh_us, 3), "expand_kernel_us": round(ex_us, 3),
+                "op_bytes": bytes_op, "op_us_events": round(op_us, 3),
+                "op_achieved_gbps": round(bytes_op / (op_us * 1e-6) / 1e9, 1),
+                "method": "HIP events on the launch stream around %d graph replays of %d launches" % (reps, L)}
+
+    out = {
+        "metric": "lora_op_us_per_layer", "value": round(us_per_layer, 3), "unit": "us/layer", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "config2 decode BGMV: 256 tokens (1/request), 64 adapters rank 16, Zipf(0.6) ids, "
+                               "4096->4096, fp16, shrink+expand; one step = this op on %d layers" % L,
+                   "layers_per_step": L, "tokens": w.T, "adapters_touched": len(used),
+                   "launch": "hip graph replay" if use_graph else "eager python launches",
+                   "tile": {"bm_shrink": plan.bm_shrink, "ksplit": plan.ksplit, "bm_expand": plan.bm_expand}},
+        "hbm_gbps": round(bytes_op / (us_per_layer * 1e-6) / 1e9, 1),
+        "hbm_frac": round(bytes_op / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(torch, w)
+    if args.all_configs:
+        bench_all_configs(torch, W, LoraPlan, dev, args.all_configs, use_graph)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

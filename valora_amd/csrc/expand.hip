@@ -23,12 +23,14 @@ namespace {
 constexpr int EXP_BN = 256;       // outputs per workgroup
 constexpr int EXP_WN = 64;        // outputs per wave
 constexpr int STAGE_LD = EXP_WN + 4;
+constexpr int EXP_MAX_BM = 256;   // tallest expand tile (tokens), one thread per token at set-up
 
 template <typename T, int KB>
 __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   __shared__ float stage[4][16][STAGE_LD];
+  __shared__ int32_t s_perm[EXP_MAX_BM];
 
   const int32_t *__restrict__ hdr = p.plan;
   const int tile_idx = blockIdx.x / p.n_ochunks;
@@ -40,33 +42,49 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lrow = lane & 15, kg = lane >> 4;
-  const int32_t *__restrict__ perm = p.plan + p.off_perm;
   const int64_t base = (int64_t)astart + (int64_t)r * p.slot;
-  const float scale = Tr::to_float(p.scales[a]);
   const int o_wave = oc * EXP_BN + wave * EXP_WN;
 
-  // B fragments: bfrag[nb][kb] = B^T[o = o_wave + nb*16 + lrow][j0 .. j0+8), j0 = kb*32 + kg*8
-  u32x4 bfrag[4][KB];
+  // Everything that depends only on the tile header is requested first, in one round trip:
+  // the tile's token indices, the pool rows of the B fragments and the scale.
+  int my_perm = 0;
+  if (tid < cnt) my_perm = p.plan[p.off_perm + pos0 + tid];
+  const float scale = Tr::to_float(p.scales[a]);
+  int64_t brow[4][KB];
+  uint32_t boff[4][KB];
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb) {
     const int o = o_wave + nb * 16 + lrow;
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
       const int j0 = kb * 32 + kg * 8;
-      u32x4 v = {0, 0, 0, 0};
+      brow[nb][kb] = -1;
+      boff[nb][kb] = 0;
       if (o < p.h_out && j0 < rk) {
         const uint32_t flat = (uint32_t)o * (uint32_t)r + (uint32_t)j0;   // < 2^16 * 2^7
         const uint32_t bin = flat / (uint32_t)p.h_out;
-        const uint32_t off = flat - bin * (uint32_t)p.h_out;
+        boff[nb][kb] = flat - bin * (uint32_t)p.h_out;
         const int64_t idx = base + bin;
-        if (idx >= 0 && idx < p.pool.a_loc_len) {
-          const int64_t row = p.pool.a_loc[idx];
-          if (row >= 0 && row < p.pool.w_rows) v = load16(p.pool.w + row * p.h_out + off);
-        }
+        if (idx >= 0 && idx < p.pool.a_loc_len) brow[nb][kb] = p.pool.a_loc[idx];
       }
-      bfrag[nb][kb] = v;
     }
   }
+  s_perm[tid] = my_perm;
+  // The only workgroup-wide barrier: it also drains the loads above (which everything below needs
+  // anyway).  No barrier may follow the bulk loads below -- a barrier waits for all outstanding
+  // global loads and would serialise the B, y and v traffic into separate round trips.
+  __syncthreads();
+
+  // B fragments: bfrag[nb][kb] = B^T[o = o_wave + nb*16 + lrow][j0 .. j0+8), j0 = kb*32 + kg*8
+  u32x4 bfrag[4][KB];
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int64_t row = brow[nb][kb];
+      bfrag[nb][kb] = (row >= 0 && row < p.pool.w_rows) ? load16(p.pool.w + row * p.h_out + boff[nb][kb])
+                                                        : u32x4{0, 0, 0, 0};
+    }
 
   // row-major roles for the y read-modify-write: 8 lanes x 16 B cover one token row of the wave's
   // 64 outputs; a wave covers 8 rows per access, two accesses per 16-token block.
@@ -75,6 +93,18 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
 
   const int n_mb = (cnt + 15) >> 4;
   for (int mb = 0; mb < n_mb; ++mb) {
+    // ---- y rows first (the longest-latency loads of the iteration)
+    u32x4 yv[2];
+    uint16_t *yp[2];
+    bool yok[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int row = mb * 16 + rr0 + 8 * h;
+      yok[h] = ocol_ok && row < cnt;
+      const int t = yok[h] ? s_perm[row] : 0;
+      yp[h] = p.y + (int64_t)t * p.h_out + o_wave + c8;
+      yv[h] = yok[h] ? load16(yp[h]) : u32x4{0, 0, 0, 0};
+    }
     // ---- v fragments: rows = tokens (lrow), 8 consecutive rank elements per lane
     const int prow = mb * 16 + lrow;
     const bool pok = prow < cnt;
@@ -86,32 +116,28 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
       if (pok && j0 < rk) {
         if (p.partial != nullptr) {
           float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          for (int s = 0; s < p.ksplit; ++s) {
-            const f32x4 *src = reinterpret_cast<const f32x4 *>(
-                p.partial + ((int64_t)s * p.T + pos0 + prow) * p.rp + j0);
-            const f32x4 lo = src[0], hi = src[1];
+          const float *src0 = p.partial + ((int64_t)pos0 + prow) * p.rp + j0;
+          const int64_t sstride = (int64_t)p.T * p.rp;
+          for (int s0 = 0; s0 < p.ksplit; s0 += 4) {   // four partials in flight at a time
+            f32x4 lo[4], hi[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) { f[i] += lo[i]; f[4 + i] += hi[i]; }
+            for (int u = 0; u < 4; ++u) {
+              const bool ok = s0 + u < p.ksplit;
+              const f32x4 *src = reinterpret_cast<const f32x4 *>(src0 + (int64_t)(s0 + u) * sstride);
+              lo[u] = ok ? src[0] : f32x4{0.f, 0.f, 0.f, 0.f};
+              hi[u] = ok ? src[1] : f32x4{0.f, 0.f, 0.f, 0.f};
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+              for (int i = 0; i < 4; ++i) { f[i] += lo[u][i]; f[4 + i] += hi[u][i]; }
           }
           v = pack8<T>(f);
         } else {
-          const int t = perm[pos0 + prow];
-          v = load16(p.xv + (int64_t)t * p.v_stride + j0);
+          v = load16(p.xv + (int64_t)s_perm[prow] * p.v_stride + j0);
         }
       }
       vfrag[kb] = v;
-    }
-    // ---- y rows (issued before the MFMAs so the loads overlap them)
-    u32x4 yv[2];
-    uint16_t *yp[2];
-    bool yok[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int row = mb * 16 + rr0 + 8 * h;
-      yok[h] = ocol_ok && row < cnt;
-      const int t = yok[h] ? perm[pos0 + row] : 0;
-      yp[h] = p.y + (int64_t)t * p.h_out + o_wave + c8;
-      yv[h] = yok[h] ? load16(yp[h]) : u32x4{0, 0, 0, 0};
     }
     // ---- delta block through the matrix cores, staged to LDS in token-major order
 #pragma unroll
@@ -123,7 +149,10 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) stage[wave][kg * 4 + i][nb * 16 + lrow] = acc[i];
     }
-    __syncthreads();
+    // stage[wave] is private to this wave and a wave's LDS operations execute in order, so only
+    // the compiler has to be kept from reordering the reads below over the writes above.
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       if (yok[h]) {
@@ -135,7 +164,8 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
         store16(yp[h], pack8<T>(f));
       }
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
   }
 }
 

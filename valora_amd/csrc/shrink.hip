@@ -69,20 +69,29 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs p) {
   const int kend = min(p.h_in, kbeg + p.kchunk);
   // The trip count must be wave-uniform: MFMA ignores EXEC, so a lane that left the loop early
   // would still feed its stale registers into the matrix core.  Lanes past the end load zeros.
-  for (int kb = kbeg + wave * 32; kb < kend; kb += 128) {
-    const int k = kb + kg * 8;
-    const bool kok = k < kend;
-    u32x4 xa[MB], wb[NB];
+  // U K-steps are loaded before any is consumed: the kernel is bound by memory latency, so what
+  // matters is how many 16-byte loads each lane has in flight (U * (MB + NB)).
+  constexpr int U = (MB + NB <= 2) ? 8 : (MB + NB <= 4) ? 4 : (MB + NB <= 8) ? 2 : 1;
+  for (int kb0 = kbeg + wave * 32; kb0 < kend; kb0 += 128 * U) {
+    u32x4 xa[U][MB], wb[U][NB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) xa[mb] = (xok[mb] && kok) ? load16(xp[mb] + k) : u32x4{0, 0, 0, 0};
+    for (int u = 0; u < U; ++u) {
+      const int k = kb0 + u * 128 + kg * 8;
+      const bool kok = k < kend;
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) wb[nb] = (wok[nb] && kok) ? load16(wp[nb] + k) : u32x4{0, 0, 0, 0};
+      for (int mb = 0; mb < MB; ++mb) xa[u][mb] = (xok[mb] && kok) ? load16(xp[mb] + k) : u32x4{0, 0, 0, 0};
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      if (nb * 16 < r) {
+      for (int nb = 0; nb < NB; ++nb) wb[u][nb] = (wok[nb] && kok) ? load16(wp[nb] + k) : u32x4{0, 0, 0, 0};
+    }
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          acc[mb][nb] = Tr::mfma(as<vec8>(xa[mb]), as<vec8>(wb[nb]), acc[mb][nb]);
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        if (nb * 16 < r) {
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            acc[mb][nb] = Tr::mfma(as<vec8>(xa[u][mb]), as<vec8>(wb[u][nb]), acc[mb][nb]);
+        }
       }
     }
   }

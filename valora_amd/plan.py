@@ -37,7 +37,7 @@ class LoraPlan:
         cfg = tile_table.lookup(self.T, self.max_rank, hidden, self.n_adapters)
         self.bm_shrink = cfg.bm_shrink if bm_shrink is None else bm_shrink
         self.bm_expand = cfg.bm_expand if bm_expand is None else bm_expand
-        self.ksplit = cfg.ksplit if ksplit is None else ksplit
+        self.ksplit = max(1, cfg.ksplit if ksplit is None else ksplit)
         L = _lib.lib()
         nbytes = int(L.mlora_plan_bytes(self.T, self.n_adapters))
         self.buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
@@ -86,6 +86,36 @@ class LoraPlan:
     def tiles_expand(self): return self._section(3)
 
     # -- the op -------------------------------------------------------------------------------------
+    def _check(self, x, y, key_buffer, value_buffer):
+        for t, w in ((x, key_buffer), (y, value_buffer)):
+            if t is None:
+                continue
+            if t.dim() != 2 or t.size(0) != self.T or not t.is_contiguous():
+                raise RuntimeError(f"x and y must be contiguous [T={self.T}, H] matrices")
+            if _lib.dtype_code(t.dtype) < 0 or w.dtype != t.dtype:
+                raise RuntimeError(f"No suitable kernel. h_in={t.size(1)} h_out={t.size(1)} dtype={t.dtype}")
+
+    def shrink(self, x: torch.Tensor, key_buffer: torch.Tensor, a_start, a_len, a_loc, slot: int) -> None:
+        """First launch of the op alone: split-K partials of ``x @ A_a.T`` into ``self.partial``."""
+        self._check(x, None, key_buffer, None)
+        pa = _lib.make_pool(key_buffer, a_start, a_len, a_loc, x.size(1), self.n_slots)
+        _lib.check(_lib.lib().mlora_shrink_partial(
+            _lib.current_stream(self.device), self.handle, _lib.ptr(self.partial), self.partial.numel() * 4,
+            _lib.ptr(x), self.T, x.size(1), self.max_rank, pa, int(slot), max(int(self.ksplit), 1),
+            _lib.dtype_code(x.dtype)))
+
+    def expand(self, y: torch.Tensor, value_buffer: torch.Tensor, a_start, a_len, a_loc, slot: int,
+               scales: torch.Tensor) -> None:
+        """Second launch alone: ``y += scale_a * T(v) @ B_a`` with v taken from ``self.partial``."""
+        self._check(None, y, None, value_buffer)
+        if scales.dtype != y.dtype:
+            scales = scales.to(y.dtype)
+        pb = _lib.make_pool(value_buffer, a_start, a_len, a_loc, y.size(1), self.n_slots)
+        _lib.check(_lib.lib().mlora_expand(
+            _lib.current_stream(self.device), self.handle, _lib.ptr(y), self.T, y.size(1), _lib.ptr(self.partial),
+            max(int(self.ksplit), 1), None, 0, self.max_rank, pb, int(slot), _lib.ptr(scales),
+            _lib.dtype_code(y.dtype)))
+
     def apply(self, y: torch.Tensor, x: torch.Tensor, key_buffer: torch.Tensor, value_buffer: torch.Tensor,
               a_start: torch.Tensor, a_len: torch.Tensor, a_loc: torch.Tensor, slot: int,
               scales: torch.Tensor) -> None:
