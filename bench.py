@@ -41,6 +41,9 @@ def parse():
     ap.add_argument("--bm-shrink", type=int, default=None)
     ap.add_argument("--bm-expand", type=int, default=None)
     ap.add_argument("--ksplit", type=int, default=None)
+    ap.add_argument("--reduce-in-expand", type=int, default=None, help="1: expand sums the split-K chunks, 0: shrink does")
+    ap.add_argument("--two-launch", action="store_true", help="shrink and expand as two launches instead of the fused kernel")
+    ap.add_argument("--replicas", type=int, default=0, help="output slices per tile of the fused kernel (0 = default)")
     ap.add_argument("--all-configs", metavar="FILE", default=None,
                     help="also measure every target of configs 1,3,4,5 and write a JSON report to FILE")
     return ap.parse_args()
@@ -199,14 +202,22 @@ def main():
     w, wd, kb, vb, xs, ys = build_layers(torch, W, dev, L)
     t = wd.targets[0]
     p = t.pool
+    if not args.two_launch and args.bm_shrink is None:
+        args.bm_shrink = 16
     plan = LoraPlan(wd.ids, p.a_start, p.a_len, 16, hidden=4096, bm_shrink=args.bm_shrink,
-                    bm_expand=args.bm_expand, ksplit=args.ksplit)
+                    bm_expand=args.bm_expand, ksplit=args.ksplit,
+                    reduce_in_expand=None if args.reduce_in_expand is None else bool(args.reduce_in_expand))
     idx = (p.a_start, p.a_len, p.a_loc)
     use_graph = not args.no_graph
 
+    fused = not args.two_launch
+
     def step():
         for l in range(L):
-            plan.apply(ys[l], xs[l], kb[l], vb[l], *idx, 0, p.a_scaling)
+            if fused:
+                plan.apply_fused(ys[l], xs[l], kb[l], vb[l], *idx, 0, p.a_scaling, args.replicas)
+            else:
+                plan.apply(ys[l], xs[l], kb[l], vb[l], *idx, 0, p.a_scaling)
 
     def shrink_only():
         for l in range(L):
@@ -253,7 +264,10 @@ def main():
     bytes_expand = r_sum * 4096 * s_el + 2 * w.T * 4096 * s_el
     bytes_op = w.algorithmic_bytes("q")
     assert bytes_op == bytes_shrink + bytes_expand
-    dom = ("expand_kernel", bytes_expand, ex_us) if ex_us >= sh_us else ("shrink_kernel", bytes_shrink, sh_us)
+    if fused:
+        dom = ("fused_kernel", bytes_op, op_us)
+    else:
+        dom = ("expand_kernel", bytes_expand, ex_us) if ex_us >= sh_us else ("shrink_kernel", bytes_shrink, sh_us)
     achieved = dom[1] / (dom[2] * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
@@ -271,6 +285,7 @@ def main():
                                "4096->4096, fp16, shrink+expand; one step = this op on %d layers" % L,
                    "layers_per_step": L, "tokens": w.T, "adapters_touched": len(used),
                    "launch": "hip graph replay" if use_graph else "eager python launches",
+                   "kernels": "fused shrink+expand, one launch" if fused else "shrink then expand, two launches",
                    "tile": {"bm_shrink": plan.bm_shrink, "ksplit": plan.ksplit, "bm_expand": plan.bm_expand}},
         "hbm_gbps": round(bytes_op / (us_per_layer * 1e-6) / 1e9, 1),
         "hbm_frac": round(bytes_op / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),

@@ -28,11 +28,19 @@ typedef enum {
   MLORA_ERR_LAUNCH = -4       /* the HIP runtime refused a launch */
 } mlora_status;
 
-/* Behaviour switches of the shrink store (see mlora_shrink_finish). */
+/* Behaviour switches of the shrink store (see mlora_shrink). */
 enum {
   MLORA_SHRINK_OVERWRITE = 0, /* y[t,:r] = v, columns >= r untouched (BGMV, bgmv_impl.cuh:36,147) */
   MLORA_SHRINK_ZERO_PAD = 1,  /* y[t,:width] = v, zero for columns >= r (Triton, lora_prefill.py:89,96-100) */
   MLORA_SHRINK_ACCUMULATE = 2 /* y[t,:r] += v (ATMM beta = 1, atmm/.../bgmv_impl.cuh:174) */
+};
+
+/* flags of mlora_shrink / mlora_expand / mlora_lora_apply */
+enum {
+  MLORA_REDUCE_IN_EXPAND = 1  /* split-K chunks are summed by the expand launch instead of by the
+                                 shrink's last workgroup: fewer dependent memory round trips for
+                                 small batches, more re-reads for large ones.  Must be given to both
+                                 launches of a pair, with the same ksplit.                        */
 };
 
 /* Pool + adapter index operands shared by all op entry points (device pointers).
@@ -65,8 +73,9 @@ int mlora_version(void);
 /* ---- sizing ------------------------------------------------------------------------------ */
 /* Bytes of a plan for T tokens and n_adapters adapters.                                       */
 size_t mlora_plan_bytes(int64_t T, int64_t n_adapters);
-/* Bytes of the fp32 split-K partial buffer the shrink writes and the expand reads.            */
-size_t mlora_partial_bytes(int64_t T, int64_t max_rank, int32_t ksplit);
+/* Bytes of the scratch buffer that carries v = x*A^T from mlora_shrink to mlora_expand (a T-typed
+ * [T, max_rank] matrix plus, for ksplit > 1, the fp32 split-K partials).                       */
+size_t mlora_scratch_bytes(int64_t T, int64_t max_rank, int32_t ksplit);
 /* Bytes of scratch the one-call entry points (dispatch_bgmv, dispatch_sgmm, prefill_*) need.
  * Replaces sgmm_tmp_size (atmm/valora/csrc/bgmv/bgmv_impl.cuh:128-132).                       */
 size_t mlora_workspace_bytes(int64_t T, int64_t n_adapters, int64_t max_rank);
@@ -104,33 +113,46 @@ int mlora_ids_from_requests(void *stream, int64_t *ids_out, const int32_t *b_sta
                             int64_t T, int64_t max_rows);
 
 /* ---- planned op: shrink / expand / fused ---------------------------------------------------- */
-/* partial[s][p][R] (fp32) = sum over K-chunk s of x[perm[p], k] * A[j, k]; p = sorted position.
+/* v[row, j] = T( sum_k x[t, k] * A_a[j, k] ) for j < r_a, fp32 accumulation, one rounding.
+ * out == NULL : v goes to `scratch` (rows in the plan's sorted order) for mlora_expand.
+ * out != NULL : the caller's matrix [T, out_stride] is written in token order; `mode` is one of
+ *               MLORA_SHRINK_* and `width` the number of columns ZERO_PAD fills.
+ * ksplit: K-chunks computed by separate workgroups (0 = library default); the last workgroup of
+ * a tile to finish sums the chunks in index order, so results do not depend on scheduling.
+ * Two launches that share one plan must not overlap in time (they share its arrival counters).
  * Kernel semantics: valora/csrc/bgmv/bgmv_impl.cuh:14-148.                                    */
-int mlora_shrink_partial(void *stream, const mlora_plan *plan, float *partial, size_t partial_bytes,
-                         const void *x, int64_t T, int64_t h_in, int64_t max_rank,
-                         const mlora_pool *pool, int32_t slot, int32_t ksplit, mlora_dtype dtype);
+int mlora_shrink(void *stream, const mlora_plan *plan, void *scratch, size_t scratch_bytes,
+                 const void *x, int64_t T, int64_t h_in, int64_t max_rank, const mlora_pool *pool,
+                 int32_t slot, int32_t ksplit, void *out, int64_t out_stride, int32_t mode,
+                 int32_t width, int32_t flags, mlora_dtype dtype);
 
-/* y[perm[p], j] (<-|+=) T(sum_s partial[s][p][j]); mode is one of MLORA_SHRINK_*; y has row
- * stride y_stride elements and `width` is the number of columns mode ZERO_PAD fills.          */
-int mlora_shrink_finish(void *stream, const mlora_plan *plan, const float *partial, void *y,
-                        int64_t T, int64_t y_stride, int64_t max_rank, int32_t ksplit,
-                        int32_t mode, int32_t width, mlora_dtype dtype);
-
-/* y[t,:] = T(y[t,:] + scale[a] * T(v[t,:r]) * B_a).  v comes either from `partial`
- * (summed over ksplit, rounded to T once -- the reference holds it as a T tensor between its
- * two launches) or, when partial == NULL, from xv (a T matrix [T, v_stride]).
+/* y[t,:] = T( y[t,:] + scale[a] * v[t,:r] * B_a ), fp32 accumulation, one rounding.
+ * v == NULL : v is read from `scratch` as written by mlora_shrink(out = NULL) -- pass that call's
+ *             ksplit and flags.
+ * v != NULL : a T matrix [T, v_stride] in token order (the reference's `delta` tensor).
  * Kernel semantics: valora/csrc/bgmv/bgmv_impl.cuh:152-207.                                   */
 int mlora_expand(void *stream, const mlora_plan *plan, void *y, int64_t T, int64_t h_out,
-                 const float *partial, int32_t ksplit, const void *xv, int64_t v_stride,
-                 int64_t max_rank, const mlora_pool *pool, int32_t slot, const void *scales,
-                 mlora_dtype dtype);
+                 const void *scratch, const void *v, int64_t v_stride, int64_t max_rank,
+                 const mlora_pool *pool, int32_t slot, const void *scales, int32_t ksplit,
+                 int32_t flags, mlora_dtype dtype);
 
-/* Shrink + expand of one target in one call (two launches, v stays in `partial`).  pool_a holds
+/* Shrink + expand of one target in one call (two launches, v stays in `scratch`).  pool_a holds
  * the A rows (row width h_in), pool_b the B rows (row width h_out); they share the index.     */
-int mlora_lora_apply(void *stream, const mlora_plan *plan, float *partial, size_t partial_bytes,
+int mlora_lora_apply(void *stream, const mlora_plan *plan, void *scratch, size_t scratch_bytes,
                      void *y, const void *x, int64_t T, int64_t h_in, int64_t h_out,
                      int64_t max_rank, const mlora_pool *pool_a, const mlora_pool *pool_b,
-                     int32_t slot, const void *scales, int32_t ksplit, mlora_dtype dtype);
+                     int32_t slot, const void *scales, int32_t ksplit, int32_t flags,
+                     mlora_dtype dtype);
+
+/* Shrink + expand of one target in ONE launch, for decode-like batches (few tokens per adapter):
+ * each workgroup recomputes v for its tile of <= 16 tokens and expands one slice of the output
+ * columns, so nothing is handed from one workgroup to another and no scratch is needed.
+ * Requires a plan built with bm_shrink = 16 and max_rank <= 64.  replicas = number of output
+ * slices per tile (0 = library default).  Same result as mlora_lora_apply.                    */
+int mlora_lora_fused(void *stream, const mlora_plan *plan, void *y, const void *x, int64_t T,
+                     int64_t h_in, int64_t h_out, int64_t max_rank, const mlora_pool *pool_a,
+                     const mlora_pool *pool_b, int32_t slot, const void *scales, int32_t replicas,
+                     mlora_dtype dtype);
 
 /* ---- the reference's entry points, one call each -------------------------------------------- */
 /* dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales)

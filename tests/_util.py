@@ -44,6 +44,16 @@ def run_plan(wd, name, **kw):
     return y
 
 
+def run_fused(wd, name, replicas=0):
+    from valora_amd.plan import LoraPlan
+    t = wd.target(name); p = t.pool
+    plan = LoraPlan(wd.ids, p.a_start, p.a_len, max_rank(wd), hidden=t.h_in, bm_shrink=16)
+    y = wd.y0[name].clone()
+    plan.apply_fused(y, wd.x[t.h_in], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot,
+                     p.a_scaling, replicas)
+    return y
+
+
 def run_sgmm(wd, name):
     from valora_amd.atmm_ops import dispatch_bgmv as dispatch_sgmm
     from valora_amd.segments import count_consecutive_requests

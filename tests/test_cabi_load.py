@@ -22,7 +22,7 @@ def _declared():
 def test_library_exports_every_declared_symbol():
     L = _lib.lib()
     names = _declared()
-    assert len(names) >= 17
+    assert len(names) >= 16
     for n in names:
         assert hasattr(L, n), n
     assert sorted(_lib.SYMBOLS) == names
@@ -33,8 +33,8 @@ def test_size_queries():
     L = _lib.lib()
     assert L.mlora_plan_bytes(0, 0) > 0
     assert L.mlora_plan_bytes(256, 64) >= (32 + 3 * 256 + 2 * 8 * (16 + 64) + 4 * 64) * 4
-    assert L.mlora_partial_bytes(256, 16, 8) == 8 * 256 * 16 * 4
-    assert L.mlora_partial_bytes(10, 8, 1) == 10 * 16 * 4       # rows padded to 16 columns
+    assert L.mlora_scratch_bytes(256, 16, 8) == 256 * 16 * 2 + 8 * 256 * 16 * 4   # v (T) + fp32 partials
+    assert L.mlora_scratch_bytes(16, 8, 1) == 16 * 16 * 2       # rows padded to 16 columns, no partials
     assert L.mlora_workspace_bytes(256, 64, 16) > L.mlora_plan_bytes(256, 64)
     assert L.mlora_plan_bytes(-1, 3) == 0
 

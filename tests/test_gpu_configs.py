@@ -9,7 +9,8 @@ import torch
 
 from oracle import lora_oracle as O
 from valora_amd import workloads as W
-from tests._util import (assert_parity, max_rank, oracle_target, run_bgmv, run_plan, run_prefill, run_sgmm)
+from tests._util import (assert_parity, max_rank, oracle_target, run_bgmv, run_fused, run_plan, run_prefill,
+                         run_sgmm)
 
 pytestmark = pytest.mark.gpu
 
@@ -35,6 +36,8 @@ def test_small_configs_all_entry_points(dev, n):
         # and y -- bf16 carries 8 significant bits, so ~1e-3 relative is the floor for any implementation
         # that, like the reference, holds v as a 16-bit tensor
         assert O.rel_l2(got, exact) <= (4e-3 if w.dtype == torch.bfloat16 else 5e-4)
+        for rep in (0, 1, 3):
+            assert_parity(run_fused(wd, t.name, rep).cpu(), want, f"config{n}/{t.name}/fused rep={rep}")
         if t.h_in == t.h_out:      # the reference's entry points decide the direction by h_in < h_out
             y, delta = run_bgmv(wd, t.name)
             assert_parity(y.cpu(), want, f"config{n}/{t.name}/bgmv")
@@ -68,10 +71,13 @@ def test_config2_full(dev, variant):
     want = oracle_target(w, "q")
     assert_parity(run_plan(wd, "q").cpu(), want, "config2/plan")
     assert_parity(run_bgmv(wd, "q")[0].cpu(), want, "config2/bgmv")
+    for rep in (0, 1, 2, 7, 64):
+        assert_parity(run_fused(wd, "q", rep).cpu(), want, f"config2/fused rep={rep}")
     for ks in (1, 4, 16):
-        for bm_s, bm_e in ((16, 16), (32, 64), (64, 256)):
-            assert_parity(run_plan(wd, "q", ksplit=ks, bm_shrink=bm_s, bm_expand=bm_e).cpu(), want,
-                          f"config2/plan ks={ks} bm={bm_s}/{bm_e}")
+        for bm_s, bm_e in ((16, 16), (32, 64), (64, 256), (128, 128)):
+            for rie in (False, True):
+                assert_parity(run_plan(wd, "q", ksplit=ks, bm_shrink=bm_s, bm_expand=bm_e, reduce_in_expand=rie).cpu(),
+                              want, f"config2/plan ks={ks} bm={bm_s}/{bm_e} reduce_in_expand={rie}")
 
 
 @pytest.mark.parametrize("n,names", [(3, ("q", "o", "up", "down")), (4, ("k", "gate", "down")),
@@ -82,8 +88,37 @@ def test_full_configs_vs_oracle(dev, n, names):
     for name in names:
         want = oracle_target(w, name)
         assert_parity(run_plan(wd, name).cpu(), want, f"config{n}/{name}/plan")
+        if n == 5:  # the decode-heavy layer also goes through the single-launch kernel
+            assert_parity(run_fused(wd, name).cpu(), want, f"config{n}/{name}/fused")
     sq = [t.name for t in w.targets if t.h_in == t.h_out][0]
     assert_parity(run_bgmv(wd, sq)[0].cpu(), oracle_target(w, sq), f"config{n}/{sq}/bgmv")
+
+
+@pytest.mark.parametrize("n,name", [(3, "q"), (3, "down"), (4, "v"), (4, "up"), (5, "o")])
+def test_full_configs_gemm_shrink_tiles(dev, n, name):
+    """The 128-token shrink tiles (weights staged through LDS) against the oracle, with and
+    without split-K."""
+    w = W.CONFIGS[n](targets=(name,))
+    wd = w.to(dev)
+    want = oracle_target(w, name)
+    for ks in (1, 3, 8):
+        for rie in (False, True):
+            assert_parity(run_plan(wd, name, bm_shrink=128, ksplit=ks, bm_expand=128, reduce_in_expand=rie).cpu(), want,
+                          f"config{n}/{name}/plan bm=128 ks={ks} reduce_in_expand={rie}")
+
+
+def test_rank128_both_shrink_kernels(dev):
+    g = torch.Generator().manual_seed(128)
+    ranks = [128, 64, 8, 128]
+    pool = W.make_pool(ranks, 1024, 1024, torch.bfloat16, g, True, std=0.02)
+    seq = [150, 3, 40, 1, 260, 17]
+    req = [0, 1, 2, 3, 3, 0]
+    wl = W._finish("r128", torch.bfloat16, req, seq, None, {"q": (pool, 2, 1024, 1024)}, g, True)
+    wd = wl.to(dev)
+    want = oracle_target(wl, "q")
+    for bm_s in (16, 32, 128):
+        for ks in (1, 4):
+            assert_parity(run_plan(wd, "q", bm_shrink=bm_s, ksplit=ks, bm_expand=64).cpu(), want, f"r128 bm={bm_s} ks={ks}")
 
 
 @pytest.mark.parametrize("n", [2, 3, 4, 5])
@@ -108,6 +143,17 @@ def test_full_size_properties(dev, n):
         base = run(wd.ids, x, y0, p.a_scaling)
         # determinism
         assert torch.equal(base, run(wd.ids, x, y0, p.a_scaling))
+        if n in (2, 5):
+            # the single-launch kernel is deterministic and token-permutation equivariant too
+            def runf(ids, xx, yy):
+                plan = LoraPlan(ids, p.a_start, p.a_len, R, hidden=t.h_in, bm_shrink=16)
+                out = yy.clone()
+                plan.apply_fused(out, xx, p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot,
+                                 p.a_scaling)
+                return out
+            fb = runf(wd.ids, x, y0)
+            assert torch.equal(fb, runf(wd.ids, x, y0))
+            assert torch.equal(runf(wd.ids[perm].contiguous(), x[perm].contiguous(), y0[perm].contiguous()), fb[perm])
         # token-permutation equivariance, bit for bit: a token's result does not depend on its tile-mates
         shuf = run(wd.ids[perm].contiguous(), x[perm].contiguous(), y0[perm].contiguous(), p.a_scaling)
         assert torch.equal(shuf, base[perm])

@@ -17,13 +17,14 @@ LIB_PATH = os.path.join(_HERE, "libmlora.so")
 
 MLORA_F16, MLORA_BF16 = 0, 1
 SHRINK_OVERWRITE, SHRINK_ZERO_PAD, SHRINK_ACCUMULATE = 0, 1, 2
+REDUCE_IN_EXPAND = 1
 
 # every symbol include/mlora.h declares
 SYMBOLS = [
-    "mlora_last_error", "mlora_version", "mlora_plan_bytes", "mlora_partial_bytes",
+    "mlora_last_error", "mlora_version", "mlora_plan_bytes", "mlora_scratch_bytes",
     "mlora_workspace_bytes", "mlora_build_plan", "mlora_count_consecutive",
-    "mlora_ids_from_segments", "mlora_ids_from_requests", "mlora_shrink_partial",
-    "mlora_shrink_finish", "mlora_expand", "mlora_lora_apply", "mlora_dispatch_bgmv",
+    "mlora_ids_from_segments", "mlora_ids_from_requests", "mlora_shrink", "mlora_expand", "mlora_lora_apply",
+    "mlora_lora_fused", "mlora_dispatch_bgmv",
     "mlora_dispatch_sgmm", "mlora_prefill_shrink", "mlora_prefill_expand",
 ]
 
@@ -53,10 +54,10 @@ def lib():
     L = ctypes.CDLL(LIB_PATH)
     L.mlora_last_error.restype = c_char_p
     L.mlora_version.restype = c_int
-    for n in ("mlora_plan_bytes", "mlora_partial_bytes", "mlora_workspace_bytes"):
+    for n in ("mlora_plan_bytes", "mlora_scratch_bytes", "mlora_workspace_bytes"):
         getattr(L, n).restype = c_size_t
     L.mlora_plan_bytes.argtypes = [c_int64, c_int64]
-    L.mlora_partial_bytes.argtypes = [c_int64, c_int64, c_int32]
+    L.mlora_scratch_bytes.argtypes = [c_int64, c_int64, c_int32]
     L.mlora_workspace_bytes.argtypes = [c_int64, c_int64, c_int64]
     L.mlora_build_plan.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_int64, c_void_p, c_void_p,
                                    c_int64, c_int32, c_int32, c_int32]
@@ -65,15 +66,16 @@ def lib():
     L.mlora_ids_from_segments.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64]
     L.mlora_ids_from_requests.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                           c_int64, c_int64]
-    L.mlora_shrink_partial.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_size_t, c_void_p, c_int64,
-                                       c_int64, c_int64, POINTER(Pool), c_int32, c_int32, c_int]
-    L.mlora_shrink_finish.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_void_p, c_int64, c_int64,
-                                      c_int64, c_int32, c_int32, c_int32, c_int]
-    L.mlora_expand.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_int64, c_int64, c_void_p, c_int32,
-                               c_void_p, c_int64, c_int64, POINTER(Pool), c_int32, c_void_p, c_int]
+    L.mlora_shrink.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_size_t, c_void_p, c_int64, c_int64,
+                               c_int64, POINTER(Pool), c_int32, c_int32, c_void_p, c_int64, c_int32, c_int32,
+                               c_int32, c_int]
+    L.mlora_expand.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_int64, c_int64, c_void_p, c_void_p,
+                               c_int64, c_int64, POINTER(Pool), c_int32, c_void_p, c_int32, c_int32, c_int]
     L.mlora_lora_apply.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_size_t, c_void_p, c_void_p,
                                    c_int64, c_int64, c_int64, c_int64, POINTER(Pool), POINTER(Pool),
-                                   c_int32, c_void_p, c_int32, c_int]
+                                   c_int32, c_void_p, c_int32, c_int32, c_int]
+    L.mlora_lora_fused.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                   POINTER(Pool), POINTER(Pool), c_int32, c_void_p, c_int32, c_int]
     L.mlora_dispatch_bgmv.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,
                                       c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t]
     L.mlora_dispatch_sgmm.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,
@@ -85,7 +87,7 @@ def lib():
     L.mlora_prefill_expand.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_void_p,
                                        c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                        c_int64, c_int64, c_int, c_void_p, c_size_t]
-    for n in SYMBOLS[5:]:
+    for n in SYMBOLS[5:]:  # everything after the size queries returns a status
         getattr(L, n).restype = c_int
     _lib = L
     return L

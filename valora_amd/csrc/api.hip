@@ -96,6 +96,17 @@ int default_ksplit(int64_t T, int64_t A, int bm, int64_t h_in) {
   return (int)ks;
 }
 
+}  // namespace
+
+size_t scratch_bytes(int64_t T, int64_t max_rank, int ksplit) {
+  const int64_t rp = partial_stride(max_rank);
+  size_t n = (size_t)align_up(T * rp * 2, 256);
+  if (ksplit > 1) n += (size_t)ksplit * (size_t)T * (size_t)rp * 4;
+  return n < 256 ? 256 : n;
+}
+
+namespace {
+
 PoolDev pool_dev(const mlora_pool *p) {
   PoolDev d;
   d.w = static_cast<const uint16_t *>(p->w);
@@ -133,18 +144,16 @@ size_t mlora_plan_bytes(int64_t T, int64_t n_adapters) {
   return (size_t)plan_layout(T, n_adapters).total_words * 4;
 }
 
-size_t mlora_partial_bytes(int64_t T, int64_t max_rank, int32_t ksplit) {
+size_t mlora_scratch_bytes(int64_t T, int64_t max_rank, int32_t ksplit) {
   if (T < 0 || max_rank < 0 || ksplit < 1) return 0;
-  size_t n = (size_t)ksplit * (size_t)T * (size_t)partial_stride(max_rank) * 4;
-  return n < 256 ? 256 : n;
+  return scratch_bytes(T, max_rank, ksplit);
 }
 
 size_t mlora_workspace_bytes(int64_t T, int64_t n_adapters, int64_t max_rank) {
   if (T < 0 || n_adapters < 0 || max_rank < 0) return 0;
   auto up = [](size_t n) { return (n + 255) & ~(size_t)255; };
   const int ks = default_ksplit(T, n_adapters, default_bm_shrink(T, n_adapters), 1 << 16);
-  return up(mlora_plan_bytes(T, n_adapters)) + up(mlora_partial_bytes(T, max_rank, ks)) +
-         up((size_t)T * 8 + 8) + 256;
+  return up(mlora_plan_bytes(T, n_adapters)) + up(scratch_bytes(T, max_rank, ks)) + up((size_t)T * 8 + 8) + 256;
 }
 
 int mlora_build_plan(void *stream, mlora_plan *plan, const int64_t *ids, int64_t T, const int64_t *a_start,
@@ -160,8 +169,8 @@ int mlora_build_plan(void *stream, mlora_plan *plan, const int64_t *ids, int64_t
   if (n_slots < 1) return fail(MLORA_ERR_INVALID, "build_plan: n_slots must be >= 1");
   if (bm_shrink == 0) bm_shrink = default_bm_shrink(T, n_adapters);
   if (bm_expand == 0) bm_expand = default_bm_expand(T, n_adapters);
-  if (bm_shrink != 16 && bm_shrink != 32 && bm_shrink != 64)
-    return fail(MLORA_ERR_NO_KERNEL, "build_plan: bm_shrink=%d not in {16,32,64}", bm_shrink);
+  if (bm_shrink != 16 && bm_shrink != 32 && bm_shrink != 64 && bm_shrink != 128)
+    return fail(MLORA_ERR_NO_KERNEL, "build_plan: bm_shrink=%d not in {16,32,64,128}", bm_shrink);
   if (bm_expand < 16 || bm_expand > 256 || (bm_expand % 16) != 0)
     return fail(MLORA_ERR_NO_KERNEL, "build_plan: bm_expand=%d not a multiple of 16 in [16,256]", bm_expand);
   const PlanLayout L = plan_layout(T, n_adapters);
@@ -206,116 +215,160 @@ int mlora_ids_from_requests(void *stream, int64_t *ids_out, const int32_t *b_sta
                                   max_rows);
 }
 
-int mlora_shrink_partial(void *stream, const mlora_plan *plan, float *partial, size_t partial_bytes, const void *x,
-                         int64_t T, int64_t h_in, int64_t max_rank, const mlora_pool *pool, int32_t slot,
-                         int32_t ksplit, mlora_dtype dtype) {
+int mlora_shrink(void *stream, const mlora_plan *plan, void *scratch, size_t scratch_nbytes, const void *x, int64_t T,
+                 int64_t h_in, int64_t max_rank, const mlora_pool *pool, int32_t slot, int32_t ksplit, void *out,
+                 int64_t out_stride, int32_t mode, int32_t width, int32_t flags, mlora_dtype dtype) {
   if (int rc = check_dtype(dtype, h_in, max_rank)) return rc;
   if (int rc = check_dims(T, h_in, max_rank, h_in, max_rank, dtype)) return rc;
   if (int rc = check_plan(plan, T, "shrink")) return rc;
   if (int rc = check_pool(pool, "shrink")) return rc;
   if (T == 0) return MLORA_OK;
-  if (!x || !partial) return fail(MLORA_ERR_INVALID, "shrink: null pointer");
-  if (!aligned16(x) || !aligned16(partial)) return fail(MLORA_ERR_INVALID, "shrink: x and partial must be 16-byte aligned");
+  if (!x || !scratch) return fail(MLORA_ERR_INVALID, "shrink: null pointer");
+  if (!aligned16(x) || !aligned16(scratch)) return fail(MLORA_ERR_INVALID, "shrink: x and scratch must be 16-byte aligned");
   if (slot < 0 || slot >= pool->n_slots) return fail(MLORA_ERR_INVALID, "shrink: slot %d outside [0,%d)", slot, pool->n_slots);
+  if (ksplit == 0) ksplit = default_ksplit(T, plan->n_adapters, plan->bm_shrink, h_in);
   if (ksplit < 1 || ksplit > 64) return fail(MLORA_ERR_INVALID, "shrink: ksplit=%d outside [1,64]", ksplit);
-  if (partial_bytes < mlora_partial_bytes(T, max_rank, ksplit))
-    return fail(MLORA_ERR_WORKSPACE, "shrink: partial buffer has %zu bytes, needs %zu", partial_bytes,
-                mlora_partial_bytes(T, max_rank, ksplit));
+  if (scratch_nbytes < scratch_bytes(T, max_rank, ksplit))
+    return fail(MLORA_ERR_WORKSPACE, "shrink: scratch has %zu bytes, needs %zu", scratch_nbytes,
+                scratch_bytes(T, max_rank, ksplit));
+  if (mode < 0 || mode > 2) return fail(MLORA_ERR_INVALID, "shrink: bad mode %d", mode);
+  if (out && (out_stride < 1 || (mode == MLORA_SHRINK_ZERO_PAD && width > out_stride)))
+    return fail(MLORA_ERR_INVALID, "shrink: width %d exceeds row stride %lld", width, (long long)out_stride);
   const PlanLayout L = plan_layout(plan->T, plan->n_adapters);
+  const int64_t rp = partial_stride(max_rank);
   ShrinkArgs a;
   a.plan = static_cast<const int32_t *>(plan->dev);
+  a.counters = static_cast<int32_t *>(plan->dev) + L.off_counters;
   a.off_perm = L.off_perm;
   a.off_tiles = L.off_tiles_s;
-  a.partial = partial;
+  a.partial = reinterpret_cast<float *>(static_cast<char *>(scratch) + align_up(T * rp * 2, 256));
   a.x = static_cast<const uint16_t *>(x);
   a.pool = pool_dev(pool);
   a.T = (int)T;
   a.h_in = (int)h_in;
-  a.rp = (int)partial_stride(max_rank);
+  a.rp = (int)rp;
   a.slot = slot;
   a.ksplit = ksplit;
   a.kchunk = (int)align_up((h_in + ksplit - 1) / ksplit, 128);
+  a.partial_only = (!out && ksplit > 1 && (flags & MLORA_REDUCE_IN_EXPAND)) ? 1 : 0;
+  if (out) {
+    a.out = static_cast<uint16_t *>(out);
+    a.out_stride = out_stride;
+    a.out_by_token = 1;
+    a.mode = mode;
+    a.width = width;
+    a.ncols = (int)(max_rank < out_stride ? max_rank : out_stride);
+  } else {
+    a.out = static_cast<uint16_t *>(scratch);
+    a.out_stride = rp;
+    a.out_by_token = 0;
+    a.mode = MLORA_SHRINK_OVERWRITE;
+    a.width = 0;
+    a.ncols = (int)rp;
+  }
   return launch_shrink((hipStream_t)stream, a, plan->bm_shrink, (int)max_rank,
                        tiles_upper(T, plan->n_adapters, plan->bm_shrink), dtype);
 }
 
-int mlora_shrink_finish(void *stream, const mlora_plan *plan, const float *partial, void *y, int64_t T,
-                        int64_t y_stride, int64_t max_rank, int32_t ksplit, int32_t mode, int32_t width,
-                        mlora_dtype dtype) {
-  if (int rc = check_dtype(dtype, 0, max_rank)) return rc;
-  if (int rc = check_plan(plan, T, "shrink_finish")) return rc;
-  if (T == 0) return MLORA_OK;
-  if (!partial || !y) return fail(MLORA_ERR_INVALID, "shrink_finish: null pointer");
-  if (mode < 0 || mode > 2) return fail(MLORA_ERR_INVALID, "shrink_finish: bad mode %d", mode);
-  if (max_rank <= 0 || max_rank > MAX_RANK) return fail(MLORA_ERR_NO_KERNEL, "shrink_finish: max_rank=%lld", (long long)max_rank);
-  if (y_stride < 1 || (mode == MLORA_SHRINK_ZERO_PAD && width > y_stride))
-    return fail(MLORA_ERR_INVALID, "shrink_finish: width %d exceeds row stride %lld", width, (long long)y_stride);
-  const PlanLayout L = plan_layout(plan->T, plan->n_adapters);
-  FinishArgs a;
-  a.plan = static_cast<const int32_t *>(plan->dev);
-  a.off_perm = L.off_perm;
-  a.off_prank = L.off_prank;
-  a.partial = partial;
-  a.y = static_cast<uint16_t *>(y);
-  a.y_stride = y_stride;
-  a.T = (int)T;
-  a.rp = (int)partial_stride(max_rank);
-  a.ncols = (int)(max_rank < y_stride ? max_rank : y_stride);
-  a.ksplit = ksplit;
-  a.mode = mode;
-  a.width = width;
-  return launch_finish((hipStream_t)stream, a, dtype);
-}
-
-int mlora_expand(void *stream, const mlora_plan *plan, void *y, int64_t T, int64_t h_out, const float *partial,
-                 int32_t ksplit, const void *xv, int64_t v_stride, int64_t max_rank, const mlora_pool *pool,
-                 int32_t slot, const void *scales, mlora_dtype dtype) {
+int mlora_expand(void *stream, const mlora_plan *plan, void *y, int64_t T, int64_t h_out, const void *scratch,
+                 const void *v, int64_t v_stride, int64_t max_rank, const mlora_pool *pool, int32_t slot,
+                 const void *scales, int32_t ksplit, int32_t flags, mlora_dtype dtype) {
   if (int rc = check_dtype(dtype, max_rank, h_out)) return rc;
   if (int rc = check_dims(T, h_out, max_rank, max_rank, h_out, dtype)) return rc;
   if (int rc = check_plan(plan, T, "expand")) return rc;
   if (int rc = check_pool(pool, "expand")) return rc;
   if (T == 0) return MLORA_OK;
   if (!y || !scales) return fail(MLORA_ERR_INVALID, "expand: null pointer");
-  if (!partial && !xv) return fail(MLORA_ERR_INVALID, "expand: neither partial nor xv given");
-  if (!aligned16(y) || !aligned16(partial) || !aligned16(xv))
-    return fail(MLORA_ERR_INVALID, "expand: y, partial and xv must be 16-byte aligned");
-  if (!partial && (v_stride < max_rank || (v_stride % 8) != 0))
+  if (!scratch && !v) return fail(MLORA_ERR_INVALID, "expand: neither scratch nor v given");
+  if (!aligned16(y) || !aligned16(scratch) || !aligned16(v))
+    return fail(MLORA_ERR_INVALID, "expand: y, scratch and v must be 16-byte aligned");
+  if (v && (v_stride < max_rank || (v_stride % 8) != 0))
     return fail(MLORA_ERR_NO_KERNEL, "No suitable kernel. h_in=%lld h_out=%lld dtype=%s", (long long)v_stride,
                 (long long)h_out, dtype_name(dtype));
   if (slot < 0 || slot >= pool->n_slots) return fail(MLORA_ERR_INVALID, "expand: slot %d outside [0,%d)", slot, pool->n_slots);
-  if (partial && (ksplit < 1 || ksplit > 64)) return fail(MLORA_ERR_INVALID, "expand: ksplit=%d outside [1,64]", ksplit);
   const PlanLayout L = plan_layout(plan->T, plan->n_adapters);
   ExpandArgs a;
   a.plan = static_cast<const int32_t *>(plan->dev);
   a.off_perm = L.off_perm;
   a.off_tiles = L.off_tiles_e;
   a.y = static_cast<uint16_t *>(y);
-  a.partial = partial;
-  a.xv = static_cast<const uint16_t *>(xv);
-  a.v_stride = v_stride;
+  a.v = static_cast<const uint16_t *>(v ? v : scratch);
+  a.v_stride = v ? v_stride : partial_stride(max_rank);
+  a.v_by_pos = v ? 0 : 1;
+  a.partial = nullptr;
+  a.ksplit = 1;
+  a.rp = (int)partial_stride(max_rank);
+  if (!v && ksplit > 1 && (flags & MLORA_REDUCE_IN_EXPAND)) {
+    if (ksplit > 64) return fail(MLORA_ERR_INVALID, "expand: ksplit=%d outside [1,64]", ksplit);
+    a.partial = reinterpret_cast<const float *>(static_cast<const char *>(scratch) + align_up(T * a.rp * 2, 256));
+    a.ksplit = ksplit;
+  }
   a.pool = pool_dev(pool);
   a.scales = static_cast<const uint16_t *>(scales);
   a.T = (int)T;
   a.h_out = (int)h_out;
-  a.rp = (int)partial_stride(max_rank);
   a.kmax = (int)max_rank;
   a.slot = slot;
-  a.ksplit = ksplit;
   a.n_ochunks = (int)((h_out + expand_bn() - 1) / expand_bn());
   return launch_expand((hipStream_t)stream, a, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand),
                        dtype);
 }
 
-int mlora_lora_apply(void *stream, const mlora_plan *plan, float *partial, size_t partial_bytes, void *y,
+int mlora_lora_apply(void *stream, const mlora_plan *plan, void *scratch, size_t scratch_nbytes, void *y,
                      const void *x, int64_t T, int64_t h_in, int64_t h_out, int64_t max_rank,
                      const mlora_pool *pool_a, const mlora_pool *pool_b, int32_t slot, const void *scales,
-                     int32_t ksplit, mlora_dtype dtype) {
+                     int32_t ksplit, int32_t flags, mlora_dtype dtype) {
   if (!plan) return fail(MLORA_ERR_INVALID, "lora_apply: plan is null");
   if (ksplit == 0) ksplit = default_ksplit(T, plan->n_adapters, plan->bm_shrink, h_in);
-  if (int rc = mlora_shrink_partial(stream, plan, partial, partial_bytes, x, T, h_in, max_rank, pool_a, slot, ksplit,
-                                    dtype))
+  if (int rc = mlora_shrink(stream, plan, scratch, scratch_nbytes, x, T, h_in, max_rank, pool_a, slot, ksplit, nullptr,
+                            0, MLORA_SHRINK_OVERWRITE, 0, flags, dtype))
     return rc;
-  return mlora_expand(stream, plan, y, T, h_out, partial, ksplit, nullptr, 0, max_rank, pool_b, slot, scales, dtype);
+  return mlora_expand(stream, plan, y, T, h_out, scratch, nullptr, 0, max_rank, pool_b, slot, scales, ksplit, flags,
+                      dtype);
+}
+
+int mlora_lora_fused(void *stream, const mlora_plan *plan, void *y, const void *x, int64_t T, int64_t h_in,
+                     int64_t h_out, int64_t max_rank, const mlora_pool *pool_a, const mlora_pool *pool_b,
+                     int32_t slot, const void *scales, int32_t replicas, mlora_dtype dtype) {
+  if (int rc = check_dtype(dtype, h_in, h_out)) return rc;
+  if (int rc = check_dims(T, h_in, max_rank, h_in, h_out, dtype)) return rc;
+  if (int rc = check_dims(T, h_out, max_rank, h_in, h_out, dtype)) return rc;
+  if (int rc = check_plan(plan, T, "lora_fused")) return rc;
+  if (int rc = check_pool(pool_a, "lora_fused")) return rc;
+  if (int rc = check_pool(pool_b, "lora_fused")) return rc;
+  if (plan->bm_shrink != 16)
+    return fail(MLORA_ERR_NO_KERNEL, "lora_fused: needs a plan built with bm_shrink=16 (has %d)", plan->bm_shrink);
+  if (max_rank > 64) return fail(MLORA_ERR_NO_KERNEL, "lora_fused: max_rank=%lld > 64 uses the two-launch path", (long long)max_rank);
+  if (T == 0) return MLORA_OK;
+  if (!y || !x || !scales) return fail(MLORA_ERR_INVALID, "lora_fused: null pointer");
+  if (!aligned16(y) || !aligned16(x)) return fail(MLORA_ERR_INVALID, "lora_fused: x and y must be 16-byte aligned");
+  if (slot < 0 || slot >= pool_a->n_slots || slot >= pool_b->n_slots)
+    return fail(MLORA_ERR_INVALID, "lora_fused: slot %d out of range", slot);
+  const int64_t tiles = tiles_upper(T, plan->n_adapters, 16);
+  const int64_t max_rep = (h_out + 63) / 64;
+  if (replicas == 0) {  // about 1.5 workgroups per compute unit
+    replicas = (int32_t)((384 + tiles - 1) / tiles);
+  }
+  if (replicas < 1) replicas = 1;
+  if (replicas > max_rep) replicas = (int32_t)max_rep;
+  const PlanLayout L = plan_layout(plan->T, plan->n_adapters);
+  FusedArgs a;
+  a.plan = static_cast<const int32_t *>(plan->dev);
+  a.off_perm = L.off_perm;
+  a.off_tiles = L.off_tiles_s;
+  a.y = static_cast<uint16_t *>(y);
+  a.x = static_cast<const uint16_t *>(x);
+  a.pa = pool_dev(pool_a);
+  a.pb = pool_dev(pool_b);
+  a.scales = static_cast<const uint16_t *>(scales);
+  a.T = (int)T;
+  a.h_in = (int)h_in;
+  a.h_out = (int)h_out;
+  a.kmax = (int)max_rank;
+  a.slot = slot;
+  a.tiles_pad = (int)align_up(tiles, 8);  // replicas of a tile land on the same XCD (workgroup id mod 8)
+  a.o_per_wg = (int)align_up((h_out + replicas - 1) / replicas, 64);
+  return launch_fused((hipStream_t)stream, a, (int)max_rank, replicas, dtype);
 }
 
 // ---- one-call entry points ------------------------------------------------------------------------
@@ -339,19 +392,17 @@ static int one_call(void *stream, void *y, const void *x, const mlora_pool *pool
     return rc;
   if (expand) {
     if (narrow_stride == 0) narrow_stride = h_in;
-    return mlora_expand(stream, &plan, y, T, h_out, nullptr, 0, x, narrow_stride, narrow, pool, (int32_t)qkvo, scales,
-                        dtype);
+    return mlora_expand(stream, &plan, y, T, h_out, nullptr, x, narrow_stride, narrow, pool, (int32_t)qkvo, scales, 1,
+                        0, dtype);
   }
   const int ksplit = default_ksplit(T, pool->n_adapters, plan.bm_shrink, h_in);
-  const size_t pbytes = mlora_partial_bytes(T, narrow, ksplit);
-  float *partial = static_cast<float *>(ws.take(pbytes));
-  if (!partial) return fail(MLORA_ERR_WORKSPACE, "%s: workspace too small (needs %zu bytes)", who,
+  const size_t sbytes = scratch_bytes(T, narrow, ksplit);
+  void *scratch = ws.take(sbytes);
+  if (!scratch) return fail(MLORA_ERR_WORKSPACE, "%s: workspace too small (needs %zu bytes)", who,
                             mlora_workspace_bytes(T, pool->n_adapters, narrow));
-  if (int rc = mlora_shrink_partial(stream, &plan, partial, pbytes, x, T, h_in, narrow, pool, (int32_t)qkvo, ksplit, dtype))
-    return rc;
   if (narrow_stride == 0) narrow_stride = h_out;
-  return mlora_shrink_finish(stream, &plan, partial, y, T, narrow_stride, narrow, ksplit, shrink_mode,
-                             shrink_width, dtype);
+  return mlora_shrink(stream, &plan, scratch, sbytes, x, T, h_in, narrow, pool, (int32_t)qkvo, ksplit, y,
+                      narrow_stride, shrink_mode, shrink_width, 0, dtype);
 }
 
 int mlora_dispatch_bgmv(void *stream, void *y, const void *x, const mlora_pool *pool, const int64_t *indicies,

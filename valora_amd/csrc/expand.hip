@@ -9,9 +9,9 @@
 // turned through a small LDS tile so that the read-modify-write of y is done with 16-byte
 // accesses of 128 contiguous bytes per token row; the add is done in fp32 and rounded once.
 //
-// v comes from the shrink's split-K partials (summed in a fixed order and rounded to T once, as
-// the reference does by holding `delta` in a T tensor between its two launches) or from a T
-// matrix supplied by the caller.
+// v is a T matrix: either the shrink's internal buffer (rows in sorted-position order; rounded
+// to T once, as the reference does by holding `delta` in a T tensor between its two launches)
+// or a matrix supplied by the caller (rows in token order).
 //
 // Reference semantics: valora/csrc/bgmv/bgmv_impl.cuh:152-207.
 #include "kernel_common.h"
@@ -25,7 +25,7 @@ constexpr int EXP_WN = 64;        // outputs per wave
 constexpr int STAGE_LD = EXP_WN + 4;
 constexpr int EXP_MAX_BM = 256;   // tallest expand tile (tokens), one thread per token at set-up
 
-template <typename T, int KB>
+template <typename T, int KB, bool PARTIAL>
 __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
@@ -114,11 +114,13 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
       const int j0 = kb * 32 + kg * 8;
       u32x4 v = {0, 0, 0, 0};
       if (pok && j0 < rk) {
-        if (p.partial != nullptr) {
+        if constexpr (PARTIAL) {
+          // split-K partials of the shrink: all chunks are requested before any is consumed,
+          // summed in chunk order and rounded to T once
           float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
           const float *src0 = p.partial + ((int64_t)pos0 + prow) * p.rp + j0;
           const int64_t sstride = (int64_t)p.T * p.rp;
-          for (int s0 = 0; s0 < p.ksplit; s0 += 4) {   // four partials in flight at a time
+          for (int s0 = 0; s0 < p.ksplit; s0 += 4) {
             f32x4 lo[4], hi[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
@@ -134,7 +136,8 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
           }
           v = pack8<T>(f);
         } else {
-          v = load16(p.xv + (int64_t)s_perm[prow] * p.v_stride + j0);
+          const int64_t vrow = p.v_by_pos ? (int64_t)(pos0 + prow) : (int64_t)s_perm[prow];
+          v = load16(p.v + vrow * p.v_stride + j0);
         }
       }
       vfrag[kb] = v;
@@ -172,9 +175,18 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
 template <typename T>
 int launch_expand_t(hipStream_t st, const ExpandArgs &a, int kb, dim3 grid) {
   switch (kb) {
-    case 1: hipLaunchKernelGGL((expand_kernel<T, 1>), grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((expand_kernel<T, 2>), grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL((expand_kernel<T, 4>), grid, dim3(256), 0, st, a); break;
+    case 1:
+      if (a.partial) hipLaunchKernelGGL((expand_kernel<T, 1, true>), grid, dim3(256), 0, st, a);
+      else hipLaunchKernelGGL((expand_kernel<T, 1, false>), grid, dim3(256), 0, st, a);
+      break;
+    case 2:
+      if (a.partial) hipLaunchKernelGGL((expand_kernel<T, 2, true>), grid, dim3(256), 0, st, a);
+      else hipLaunchKernelGGL((expand_kernel<T, 2, false>), grid, dim3(256), 0, st, a);
+      break;
+    case 4:
+      if (a.partial) hipLaunchKernelGGL((expand_kernel<T, 4, true>), grid, dim3(256), 0, st, a);
+      else hipLaunchKernelGGL((expand_kernel<T, 4, false>), grid, dim3(256), 0, st, a);
+      break;
     default: return fail(MLORA_ERR_NO_KERNEL, "expand: no kernel for %d rank blocks", kb);
   }
   return check_launch("expand_kernel");

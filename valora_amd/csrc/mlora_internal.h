@@ -10,11 +10,12 @@ namespace mlora {
 
 // ---- plan buffer layout (int32 words) ------------------------------------------------------
 //   hdr[32] | perm[T] | padapter[T] | prank[T] | tiles_s[max_tiles][8] | tiles_e[max_tiles][8]
-//   | scratch: cnt[A] gstart[A] toff_s[A] toff_e[A]
+//   | counters[max_tiles] | scratch: cnt[A] gstart[A] toff_s[A] toff_e[A]
 // perm[p]     token index at sorted position p (tokens grouped by adapter, original order kept
 //             inside a group); positions >= hdr[H_NACTIVE] are unused
 // padapter[p] adapter of position p;  prank[p] its rank
 // tile        {adapter, rank, first position, token count, a_start[adapter], 0, 0, 0}
+// counters[i] split-K arrival counter of shrink tile i; zero between launches
 constexpr int HDR_WORDS = 32;
 constexpr int TILE_WORDS = 8;
 constexpr int32_t PLAN_MAGIC = 0x4d4c5241;
@@ -31,7 +32,7 @@ constexpr int MAX_RANK = 128;
 
 struct PlanLayout {
   int64_t T, A, max_tiles;
-  int64_t off_perm, off_padapter, off_prank, off_tiles_s, off_tiles_e, off_scratch, total_words;
+  int64_t off_perm, off_padapter, off_prank, off_tiles_s, off_tiles_e, off_counters, off_scratch, total_words;
 };
 
 static inline __host__ __device__ int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
@@ -46,7 +47,8 @@ static inline PlanLayout plan_layout(int64_t T, int64_t A) {
   L.off_prank = align_up(L.off_padapter + T, 8);
   L.off_tiles_s = align_up(L.off_prank + T, 8);
   L.off_tiles_e = L.off_tiles_s + L.max_tiles * TILE_WORDS;
-  L.off_scratch = L.off_tiles_e + L.max_tiles * TILE_WORDS;
+  L.off_counters = L.off_tiles_e + L.max_tiles * TILE_WORDS;
+  L.off_scratch = align_up(L.off_counters + L.max_tiles, 8);
   L.total_words = L.off_scratch + 4 * A + 8;
   return L;
 }
@@ -72,36 +74,47 @@ struct PoolDev {
 
 struct ShrinkArgs {
   const int32_t *plan;
+  int32_t *counters;          // plan + off_counters
   int64_t off_perm, off_tiles;
-  float *partial;
+  float *partial;             // [ksplit][T][rp] fp32, used when ksplit > 1
   const uint16_t *x;
   PoolDev pool;
+  uint16_t *out;              // v: [T positions][out_stride] or the caller's y: [T tokens][out_stride]
+  int64_t out_stride;
   int T, h_in, rp, slot, ksplit, kchunk;
+  int out_by_token, mode, width, ncols;
+  int partial_only;           // leave the K-chunk partials for the expand to sum (no counters, no v)
 };
 
 struct ExpandArgs {
   const int32_t *plan;
   int64_t off_perm, off_tiles;
   uint16_t *y;
-  const float *partial;
-  const uint16_t *xv;
+  const uint16_t *v;          // narrow operand, T dtype
   int64_t v_stride;
+  int v_by_pos;               // rows indexed by sorted position (internal buffer) or by token
+  const float *partial;       // when set: v = T(sum_s partial[s][pos][:]) with ksplit chunks of T*rp floats
+  int ksplit, rp;
   PoolDev pool;
   const uint16_t *scales;
-  int T, h_out, rp, kmax, slot, ksplit, n_ochunks;
+  int T, h_out, kmax, slot, n_ochunks;
 };
 
-struct FinishArgs {
+struct FusedArgs {
   const int32_t *plan;
-  int64_t off_perm, off_prank;
-  const float *partial;
+  int64_t off_perm, off_tiles;
   uint16_t *y;
-  int64_t y_stride;
-  int T, rp, ncols, ksplit, mode, width;
+  const uint16_t *x;
+  PoolDev pa, pb;
+  const uint16_t *scales;
+  int T, h_in, h_out, kmax, slot, tiles_pad, o_per_wg;
 };
 
+int launch_fused(hipStream_t st, const FusedArgs &a, int max_rank, int replicas, mlora_dtype dt);
+int fused_bn();
 int launch_plan(hipStream_t st, int32_t *plan, const PlanLayout &L, const int64_t *ids,
                 const int64_t *a_start, const int64_t *a_len, int n_slots, int bm_s, int bm_e);
+size_t scratch_bytes(int64_t T, int64_t max_rank, int ksplit);
 int launch_count_consecutive(hipStream_t st, const int64_t *lora_rank, int64_t n_adapters,
                              const int64_t *indicies, int64_t T, int64_t *output_counts,
                              int64_t *rank_counts, int64_t *lora_ids, int64_t *start_ids,
@@ -114,7 +127,6 @@ int launch_ids_from_requests(hipStream_t st, int64_t *ids_out, const int32_t *b_
                              int64_t T, int64_t max_rows);
 int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int64_t grid_tiles,
                   mlora_dtype dt);
-int launch_finish(hipStream_t st, const FinishArgs &a, mlora_dtype dt);
 int launch_expand(hipStream_t st, const ExpandArgs &a, int max_rank, int64_t grid_tiles,
                   mlora_dtype dt);
 

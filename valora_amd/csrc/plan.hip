@@ -51,7 +51,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
     int32_t *__restrict__ plan, const int64_t *__restrict__ ids, const int64_t *__restrict__ a_start,
     const int64_t *__restrict__ a_len, int T, int A, int n_slots, int bm_s, int bm_e, int W,
     int64_t off_perm, int64_t off_padapter, int64_t off_prank, int64_t off_tiles_s,
-    int64_t off_tiles_e, int64_t off_scratch) {
+    int64_t off_tiles_e, int64_t off_counters, int64_t off_scratch, int max_tiles) {
   __shared__ int32_t whist[HIST_WORDS];
   __shared__ int wsum[PLAN_WAVES + 1];
   __shared__ int s_maxrank;
@@ -67,6 +67,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
   int32_t *toff_e = toff_s + A;
 
   for (int i = tid; i < W * A; i += PLAN_THREADS) whist[i] = 0;
+  for (int i = tid; i < max_tiles; i += PLAN_THREADS) plan[off_counters + i] = 0;
   if (tid == 0) { s_maxrank = 0; s_err = 0; }
   __syncthreads();
 
@@ -273,7 +274,7 @@ int launch_plan(hipStream_t st, int32_t *plan, const PlanLayout &L, const int64_
   if (W < 1) return fail(MLORA_ERR_NO_KERNEL, "plan: more than %lld adapters", (long long)MAX_ADAPTERS);
   hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(PLAN_THREADS), 0, st, plan, ids, a_start, a_len,
                      (int)L.T, A, n_slots, bm_s, bm_e, W, L.off_perm, L.off_padapter, L.off_prank,
-                     L.off_tiles_s, L.off_tiles_e, L.off_scratch);
+                     L.off_tiles_s, L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles);
   return check_launch("plan_kernel");
 }
 

@@ -5,8 +5,8 @@ The reference rebuilds its segment tensors once per forward
 (valora/server/router/model_infer/model_rpc.py:381) and then issues 8 op launches per layer with
 the same per-token ids (valora/models/peft/lora_unordered_batch_infer.py:946-988,1611-1622);
 ``LoraPlan`` is that once-per-forward object for the gfx950 kernels.  The intermediate
-``v = x @ A.T`` never becomes a caller-visible tensor: it lives in an fp32 split-K buffer between
-the two launches and is rounded to the operand dtype exactly once, where the reference stores
+``v = x @ A.T`` never becomes a caller-visible tensor: it lives in the plan's scratch buffer
+between the two launches, rounded to the operand dtype exactly once -- where the reference stores
 its ``delta`` tensor.
 """
 from __future__ import annotations
@@ -21,7 +21,8 @@ from . import _lib, tile_table
 class LoraPlan:
     def __init__(self, ids: torch.Tensor, a_start: torch.Tensor, a_len: torch.Tensor, max_rank: int,
                  n_slots: int = 4, hidden: int = 4096, bm_shrink: Optional[int] = None,
-                 bm_expand: Optional[int] = None, ksplit: Optional[int] = None):
+                 bm_expand: Optional[int] = None, ksplit: Optional[int] = None,
+                 reduce_in_expand: Optional[bool] = None):
         """``ids``: int64 per-token adapter index (negative = no adapter); ``a_start`` / ``a_len``:
         the pool index (``a_len = n_slots * rank``); ``max_rank``: widest rank among the resident
         adapters (the reference's ``max_lora_dim``, lora_unordered_batch_infer.py:181-182)."""
@@ -38,6 +39,8 @@ class LoraPlan:
         self.bm_shrink = cfg.bm_shrink if bm_shrink is None else bm_shrink
         self.bm_expand = cfg.bm_expand if bm_expand is None else bm_expand
         self.ksplit = max(1, cfg.ksplit if ksplit is None else ksplit)
+        rie = cfg.reduce_in_expand if reduce_in_expand is None else reduce_in_expand
+        self.flags = _lib.REDUCE_IN_EXPAND if rie else 0
         L = _lib.lib()
         nbytes = int(L.mlora_plan_bytes(self.T, self.n_adapters))
         self.buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
@@ -46,8 +49,8 @@ class LoraPlan:
         _lib.check(L.mlora_build_plan(_lib.current_stream(self.device), self.handle, _lib.ptr(ids.contiguous()),
                                       self.T, _lib.ptr(a_start), _lib.ptr(a_len), self.n_adapters, n_slots,
                                       self.bm_shrink, self.bm_expand))
-        pbytes = int(L.mlora_partial_bytes(self.T, self.max_rank, max(self.ksplit, 1)))
-        self.partial = torch.empty(pbytes // 4, dtype=torch.float32, device=self.device)
+        sbytes = int(L.mlora_scratch_bytes(self.T, self.max_rank, self.ksplit))
+        self.scratch = torch.empty(sbytes, dtype=torch.uint8, device=self.device)
 
     # -- introspection (synchronises; for tests and diagnostics) --------------------------------
     def header(self) -> dict:
@@ -96,25 +99,39 @@ class LoraPlan:
                 raise RuntimeError(f"No suitable kernel. h_in={t.size(1)} h_out={t.size(1)} dtype={t.dtype}")
 
     def shrink(self, x: torch.Tensor, key_buffer: torch.Tensor, a_start, a_len, a_loc, slot: int) -> None:
-        """First launch of the op alone: split-K partials of ``x @ A_a.T`` into ``self.partial``."""
+        """First launch of the op alone: ``v = x @ A_a.T`` into ``self.scratch``."""
         self._check(x, None, key_buffer, None)
         pa = _lib.make_pool(key_buffer, a_start, a_len, a_loc, x.size(1), self.n_slots)
-        _lib.check(_lib.lib().mlora_shrink_partial(
-            _lib.current_stream(self.device), self.handle, _lib.ptr(self.partial), self.partial.numel() * 4,
-            _lib.ptr(x), self.T, x.size(1), self.max_rank, pa, int(slot), max(int(self.ksplit), 1),
-            _lib.dtype_code(x.dtype)))
+        _lib.check(_lib.lib().mlora_shrink(
+            _lib.current_stream(self.device), self.handle, _lib.ptr(self.scratch), self.scratch.numel(),
+            _lib.ptr(x), self.T, x.size(1), self.max_rank, pa, int(slot), int(self.ksplit), None, 0, 0, 0,
+            self.flags, _lib.dtype_code(x.dtype)))
 
     def expand(self, y: torch.Tensor, value_buffer: torch.Tensor, a_start, a_len, a_loc, slot: int,
                scales: torch.Tensor) -> None:
-        """Second launch alone: ``y += scale_a * T(v) @ B_a`` with v taken from ``self.partial``."""
+        """Second launch alone: ``y += scale_a * v @ B_a`` with v taken from ``self.scratch``."""
         self._check(None, y, None, value_buffer)
         if scales.dtype != y.dtype:
             scales = scales.to(y.dtype)
         pb = _lib.make_pool(value_buffer, a_start, a_len, a_loc, y.size(1), self.n_slots)
         _lib.check(_lib.lib().mlora_expand(
-            _lib.current_stream(self.device), self.handle, _lib.ptr(y), self.T, y.size(1), _lib.ptr(self.partial),
-            max(int(self.ksplit), 1), None, 0, self.max_rank, pb, int(slot), _lib.ptr(scales),
+            _lib.current_stream(self.device), self.handle, _lib.ptr(y), self.T, y.size(1), _lib.ptr(self.scratch),
+            None, 0, self.max_rank, pb, int(slot), _lib.ptr(scales), int(self.ksplit), self.flags,
             _lib.dtype_code(y.dtype)))
+
+    def apply_fused(self, y: torch.Tensor, x: torch.Tensor, key_buffer: torch.Tensor, value_buffer: torch.Tensor,
+                    a_start: torch.Tensor, a_len: torch.Tensor, a_loc: torch.Tensor, slot: int,
+                    scales: torch.Tensor, replicas: int = 0) -> None:
+        """Same result as ``apply`` in a single launch (plan must have ``bm_shrink == 16``)."""
+        self._check(x, y, key_buffer, value_buffer)
+        if scales.dtype != x.dtype:
+            scales = scales.to(x.dtype)
+        h_in, h_out = x.size(1), y.size(1)
+        pa = _lib.make_pool(key_buffer, a_start, a_len, a_loc, h_in, self.n_slots)
+        pb = _lib.make_pool(value_buffer, a_start, a_len, a_loc, h_out, self.n_slots)
+        _lib.check(_lib.lib().mlora_lora_fused(
+            _lib.current_stream(self.device), self.handle, _lib.ptr(y), _lib.ptr(x), self.T, h_in, h_out,
+            self.max_rank, pa, pb, int(slot), _lib.ptr(scales), int(replicas), _lib.dtype_code(x.dtype)))
 
     def apply(self, y: torch.Tensor, x: torch.Tensor, key_buffer: torch.Tensor, value_buffer: torch.Tensor,
               a_start: torch.Tensor, a_len: torch.Tensor, a_loc: torch.Tensor, slot: int,
@@ -133,6 +150,6 @@ class LoraPlan:
         pa = _lib.make_pool(key_buffer, a_start, a_len, a_loc, h_in, self.n_slots)
         pb = _lib.make_pool(value_buffer, a_start, a_len, a_loc, h_out, self.n_slots)
         _lib.check(_lib.lib().mlora_lora_apply(
-            _lib.current_stream(self.device), self.handle, _lib.ptr(self.partial), self.partial.numel() * 4,
+            _lib.current_stream(self.device), self.handle, _lib.ptr(self.scratch), self.scratch.numel(),
             _lib.ptr(y), _lib.ptr(x), self.T, h_in, h_out, self.max_rank, pa, pb, int(slot), _lib.ptr(scales),
-            int(self.ksplit), code))
+            int(self.ksplit), self.flags, code))

@@ -25,9 +25,10 @@ ADAPTER_BUCKETS = (1, 8, 32, 128, 8192)
 
 @dataclass(frozen=True)
 class TileConfig:
-    bm_shrink: int   # tokens per shrink tile: 16, 32 or 64
+    bm_shrink: int   # tokens per shrink tile: 16, 32, 64 (direct loads) or 128 (weights staged in LDS)
     ksplit: int      # K-chunks the shrink is split into (partials summed by the consumer)
     bm_expand: int   # tokens per expand tile: multiple of 16 up to 256
+    reduce_in_expand: bool = False  # split-K chunks summed by the expand launch (small batches)
 
 
 def _bucket(v: int, buckets) -> int:
@@ -48,7 +49,7 @@ def fallback(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> Tile
     tiles = max(1, min(n_tokens, -(-n_tokens // bm_s) + min(n_adapters, n_tokens)))
     ksplit = max(1, min(16, hidden // 256, -(-1024 // tiles)))
     bm_e = 32 if n_tokens <= 1024 else 64 if n_tokens <= 8192 else 128
-    return TileConfig(bm_s, ksplit, bm_e)
+    return TileConfig(bm_s, ksplit, bm_e, n_tokens <= 1024)
 
 
 _table: Dict[str, TileConfig] = {}
@@ -62,7 +63,8 @@ def _load() -> None:
         with open(TABLE_PATH) as f:
             raw = json.load(f)
         for k, v in raw.get("entries", {}).items():
-            _table[k] = TileConfig(int(v["bm_shrink"]), int(v["ksplit"]), int(v["bm_expand"]))
+            _table[k] = TileConfig(int(v["bm_shrink"]), int(v["ksplit"]), int(v["bm_expand"]),
+                                   bool(v.get("reduce_in_expand", False)))
 
 
 def lookup(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> TileConfig:
@@ -72,5 +74,5 @@ def lookup(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> TileCo
     if cfg is None:
         return fallback(n_tokens, max_rank, hidden, n_adapters)
     if max_rank > 64 and cfg.bm_shrink > 32:
-        cfg = TileConfig(32, cfg.ksplit, cfg.bm_expand)
+        cfg = TileConfig(32, cfg.ksplit, cfg.bm_expand, cfg.reduce_in_expand)
     return cfg
