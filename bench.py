@@ -42,7 +42,7 @@ def parse():
     ap.add_argument("--bm-expand", type=int, default=None)
     ap.add_argument("--ksplit", type=int, default=None)
     ap.add_argument("--reduce-in-expand", type=int, default=None, help="1: expand sums the split-K chunks, 0: shrink does")
-    ap.add_argument("--two-launch", action="store_true", help="shrink and expand as two launches instead of the fused kernel")
+    ap.add_argument("--fused", action="store_true", help="use the single-launch fused kernel instead of shrink + expand")
     ap.add_argument("--replicas", type=int, default=0, help="output slices per tile of the fused kernel (0 = default)")
     ap.add_argument("--all-configs", metavar="FILE", default=None,
                     help="also measure every target of configs 1,3,4,5 and write a JSON report to FILE")
@@ -202,7 +202,7 @@ def main():
     w, wd, kb, vb, xs, ys = build_layers(torch, W, dev, L)
     t = wd.targets[0]
     p = t.pool
-    if not args.two_launch and args.bm_shrink is None:
+    if args.fused and args.bm_shrink is None:
         args.bm_shrink = 16
     plan = LoraPlan(wd.ids, p.a_start, p.a_len, 16, hidden=4096, bm_shrink=args.bm_shrink,
                     bm_expand=args.bm_expand, ksplit=args.ksplit,
@@ -210,7 +210,7 @@ def main():
     idx = (p.a_start, p.a_len, p.a_loc)
     use_graph = not args.no_graph
 
-    fused = not args.two_launch
+    fused = args.fused
 
     def step():
         for l in range(L):
