@@ -37,10 +37,10 @@ enum {
 
 /* flags of mlora_shrink / mlora_expand / mlora_lora_apply */
 enum {
-  MLORA_REDUCE_IN_EXPAND = 1  /* split-K chunks are summed by the expand launch instead of by the
-                                 shrink's last workgroup: fewer dependent memory round trips for
-                                 small batches, more re-reads for large ones.  Must be given to both
-                                 launches of a pair, with the same ksplit.                        */
+  MLORA_REDUCE_IN_EXPAND = 1  /* split-K chunks are summed by the expand launch instead of by a
+                                 separate reduce launch: one launch fewer for small batches, more
+                                 re-reads for large ones.  Must be given to both launches of a pair,
+                                 with the same ksplit.                                            */
 };
 
 /* Pool + adapter index operands shared by all op entry points (device pointers).
@@ -117,9 +117,9 @@ int mlora_ids_from_requests(void *stream, int64_t *ids_out, const int32_t *b_sta
  * out == NULL : v goes to `scratch` (rows in the plan's sorted order) for mlora_expand.
  * out != NULL : the caller's matrix [T, out_stride] is written in token order; `mode` is one of
  *               MLORA_SHRINK_* and `width` the number of columns ZERO_PAD fills.
- * ksplit: K-chunks computed by separate workgroups (0 = library default); the last workgroup of
- * a tile to finish sums the chunks in index order, so results do not depend on scheduling.
- * Two launches that share one plan must not overlap in time (they share its arrival counters).
+ * ksplit: K-chunks computed by separate workgroups (0 = library default); the chunks are summed
+ * in index order by a small second launch (or by mlora_expand, see MLORA_REDUCE_IN_EXPAND), so
+ * results do not depend on scheduling.
  * Kernel semantics: valora/csrc/bgmv/bgmv_impl.cuh:14-148.                                    */
 int mlora_shrink(void *stream, const mlora_plan *plan, void *scratch, size_t scratch_bytes,
                  const void *x, int64_t T, int64_t h_in, int64_t max_rank, const mlora_pool *pool,

@@ -238,9 +238,9 @@ int mlora_shrink(void *stream, const mlora_plan *plan, void *scratch, size_t scr
   const int64_t rp = partial_stride(max_rank);
   ShrinkArgs a;
   a.plan = static_cast<const int32_t *>(plan->dev);
-  a.counters = static_cast<int32_t *>(plan->dev) + L.off_counters;
   a.off_perm = L.off_perm;
   a.off_tiles = L.off_tiles_s;
+  a.off_prank = L.off_prank;
   a.partial = reinterpret_cast<float *>(static_cast<char *>(scratch) + align_up(T * rp * 2, 256));
   a.x = static_cast<const uint16_t *>(x);
   a.pool = pool_dev(pool);
@@ -266,8 +266,11 @@ int mlora_shrink(void *stream, const mlora_plan *plan, void *scratch, size_t scr
     a.width = 0;
     a.ncols = (int)rp;
   }
-  return launch_shrink((hipStream_t)stream, a, plan->bm_shrink, (int)max_rank,
-                       tiles_upper(T, plan->n_adapters, plan->bm_shrink), dtype);
+  if (int rc = launch_shrink((hipStream_t)stream, a, plan->bm_shrink, (int)max_rank,
+                             tiles_upper(T, plan->n_adapters, plan->bm_shrink), dtype))
+    return rc;
+  if (ksplit > 1 && !a.partial_only) return launch_shrink_reduce((hipStream_t)stream, a, dtype);
+  return MLORA_OK;
 }
 
 int mlora_expand(void *stream, const mlora_plan *plan, void *y, int64_t T, int64_t h_out, const void *scratch,

@@ -22,6 +22,38 @@ __device__ __forceinline__ To as(const From &v) {
 __device__ __forceinline__ u32x4 load16(const uint16_t *p) { return *reinterpret_cast<const u32x4 *>(p); }
 __device__ __forceinline__ void store16(uint16_t *p, u32x4 v) { *reinterpret_cast<u32x4 *>(p) = v; }
 
+// Direct global -> LDS load: each active lane copies 16 bytes from its own global address to
+// lds_base + lane*16 (lds_base is wave-uniform); completion is tracked by vmcnt.
+#define GLOBAL_PTR(p) (reinterpret_cast<const __attribute__((address_space(1))) void *>(reinterpret_cast<uintptr_t>(p)))
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+
+// wait until at most N vector-memory loads of this wave are outstanding (loads retire in order)
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// LDS accesses the compiler does not see as LDS accesses.  Around direct-to-LDS loads the
+// compiler's own wait insertion is conservative (it drains ALL outstanding loads before any LDS
+// access that might alias their destination), which would serialise a multi-stage ring; with
+// these the kernel orders things itself: wait_vmcnt<N>() before reading a stage,
+// wait_lgkmcnt0() + pin() before using what lds_read16 returned.
+__device__ __forceinline__ uint32_t lds_offset(const void *p) {
+  return (uint32_t)(uintptr_t)LDS_PTR(const_cast<void *>(p));
+}
+__device__ __forceinline__ u32x4 lds_read16(uint32_t off) {
+  u32x4 v;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(off) : "memory");
+  return v;
+}
+__device__ __forceinline__ void lds_write16(uint32_t off, u32x4 v) {
+  asm volatile("ds_write_b128 %0, %1" ::"v"(off), "v"(v) : "memory");
+}
+// makes v "produced here" for the compiler, so nothing that uses it moves above a preceding wait
+__device__ __forceinline__ void pin(u32x4 &v) { asm volatile("" : "+v"(v)); }
+
 template <typename T>
 struct Traits;
 

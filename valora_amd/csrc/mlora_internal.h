@@ -15,7 +15,7 @@ namespace mlora {
 //             inside a group); positions >= hdr[H_NACTIVE] are unused
 // padapter[p] adapter of position p;  prank[p] its rank
 // tile        {adapter, rank, first position, token count, a_start[adapter], 0, 0, 0}
-// counters[i] split-K arrival counter of shrink tile i; zero between launches
+// counters[i] reserved (zeroed by the plan kernel)
 constexpr int HDR_WORDS = 32;
 constexpr int TILE_WORDS = 8;
 constexpr int32_t PLAN_MAGIC = 0x4d4c5241;
@@ -74,8 +74,7 @@ struct PoolDev {
 
 struct ShrinkArgs {
   const int32_t *plan;
-  int32_t *counters;          // plan + off_counters
-  int64_t off_perm, off_tiles;
+  int64_t off_perm, off_tiles, off_prank;
   float *partial;             // [ksplit][T][rp] fp32, used when ksplit > 1
   const uint16_t *x;
   PoolDev pool;
@@ -83,7 +82,7 @@ struct ShrinkArgs {
   int64_t out_stride;
   int T, h_in, rp, slot, ksplit, kchunk;
   int out_by_token, mode, width, ncols;
-  int partial_only;           // leave the K-chunk partials for the expand to sum (no counters, no v)
+  int partial_only;           // leave the K-chunk partials for the expand to sum (no reduce launch)
 };
 
 struct ExpandArgs {
@@ -127,6 +126,7 @@ int launch_ids_from_requests(hipStream_t st, int64_t *ids_out, const int32_t *b_
                              int64_t T, int64_t max_rows);
 int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int64_t grid_tiles,
                   mlora_dtype dt);
+int launch_shrink_reduce(hipStream_t st, const ShrinkArgs &a, mlora_dtype dt);
 int launch_expand(hipStream_t st, const ExpandArgs &a, int max_rank, int64_t grid_tiles,
                   mlora_dtype dt);
 

@@ -9,10 +9,8 @@
 // several K-steps are loaded before any is consumed (the kernel is latency bound: what counts
 // is the number of 16-byte loads in flight per lane).
 //
-// Split-K without atomics on data: every workgroup writes its fp32 partial tile, then bumps a
-// per-tile counter in the plan; the workgroup that arrives last sums the `ksplit` partials in
-// index order (so the result does not depend on which one was last), rounds once to T and
-// stores v.  No workgroup ever waits for another, and the counter is reset for the next launch.
+// Split-K without atomics: every workgroup writes its fp32 partial tile and is done; the chunks
+// are summed in index order (bit-reproducible) by shrink_reduce_kernel or by the expand.
 //
 // Reference semantics: valora/csrc/bgmv/bgmv_impl.cuh:14-148 (per-token gather mat-vec with the
 // rank rows gathered through loc_indicies, fp32 accumulation, one T store per output).
@@ -43,16 +41,16 @@ __device__ __forceinline__ void store_v(const ShrinkArgs &p, int pos, int t, int
 // Epilogue shared by both shrink kernels.  `tile` is the workgroup's fp32 result in LDS, row-major
 // with row stride ld: rows = tokens of the tile, columns = rank.
 //   ksplit == 1 : rounded to T and stored.
-//   ksplit  > 1 : stored as this K-chunk's partial; the last workgroup of the tile to get here sums
-//                 the ksplit partials in index order (the result does not depend on which one was
-//                 last) and stores v.
-// The partials are written with device-scope stores and read back with device-scope loads, two
-// floats at a time, so they never rely on an XCD's L2 being written back or invalidated: a full
-// device-scope fence would flush and invalidate the whole L2 of the XCD once per workgroup
-// (measured: 5-10x slower kernels).  __syncthreads() waits until the stores are acknowledged.
+//   ksplit  > 1 : stored as this K-chunk's fp32 partial (ordinary stores, then the workgroup is
+//                 done); a later launch on the stream -- shrink_reduce_kernel, or the expand
+//                 itself for small batches -- sums the chunks in index order and rounds once.
+// An in-kernel hand-off (last workgroup of a tile sums the chunks, found through an atomic
+// counter) was measured and dropped: on this multi-XCD part it needs device-scope stores, an
+// atomic and device-scope loads, i.e. three to four dependent memory round trips at the end of
+// every workgroup (+14 us on a 30 us kernel); a device-scope fence instead made it 5-10x slower.
 template <typename T>
-__device__ __forceinline__ void shrink_epilogue(const ShrinkArgs &p, const float *tile, int ld, int tile_idx, int s,
-                                                int pos0, int cnt, int r, const int32_t *perm, int *s_last) {
+__device__ __forceinline__ void shrink_epilogue(const ShrinkArgs &p, const float *tile, int ld, int s, int pos0,
+                                                int cnt, int r, const int32_t *perm) {
   const int tid = threadIdx.x;
   if (p.ksplit == 1) {
     const int n_el = cnt * p.rp;
@@ -62,59 +60,42 @@ __device__ __forceinline__ void shrink_epilogue(const ShrinkArgs &p, const float
     }
     return;
   }
-  const int half = p.rp >> 1;          // rp is a multiple of 16
-  const int n_pair = cnt * half;
-  if (p.partial_only) {
-    // the next launch on the stream sums the chunks: ordinary stores, no counters
-    float2 *part = reinterpret_cast<float2 *>(p.partial + ((int64_t)s * p.T + pos0) * p.rp);
-    for (int e = tid; e < n_pair; e += 256) {
-      const int row = e / half, c2 = e - row * half;
-      part[e] = make_float2(tile[row * ld + 2 * c2], tile[row * ld + 2 * c2 + 1]);
-    }
-    return;
+  const int quarter = p.rp >> 2;       // rp is a multiple of 16
+  const int n_vec = cnt * quarter;
+  f32x4 *part = reinterpret_cast<f32x4 *>(p.partial + ((int64_t)s * p.T + pos0) * p.rp);
+  for (int e = tid; e < n_vec; e += 256) {
+    const int row = e / quarter, c4 = e - row * quarter;
+    const float *src = tile + row * ld + 4 * c4;
+    part[e] = f32x4{src[0], src[1], src[2], src[3]};
   }
-  {
-    unsigned long long *part = reinterpret_cast<unsigned long long *>(p.partial + ((int64_t)s * p.T + pos0) * p.rp);
-    for (int e = tid; e < n_pair; e += 256) {
-      const int row = e / half, c2 = e - row * half;
-      const float2 v = make_float2(tile[row * ld + 2 * c2], tile[row * ld + 2 * c2 + 1]);
-      __hip_atomic_store(part + e, __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED,
-                         __HIP_MEMORY_SCOPE_AGENT);
-    }
-  }
-  __syncthreads();
-  if (tid == 0) {
-    const int prev = atomicAdd(p.counters + tile_idx, 1);
-    *s_last = (prev == p.ksplit - 1);
-  }
-  __syncthreads();
-  if (!*s_last) return;
-  const unsigned long long *src = reinterpret_cast<const unsigned long long *>(p.partial + (int64_t)pos0 * p.rp);
-  const int64_t sstride = (int64_t)p.T * half;
-  for (int e = tid; e < n_pair; e += 256) {
-    const int row = e / half, c2 = e - row * half;
-    float2 v = make_float2(0.f, 0.f);
-    // eight partials are requested before any is consumed (each is a round trip to memory);
-    // the sum itself runs in index order
+}
+
+// v[row, :] = T(sum_s partial[s][row][:]) for every row that has an adapter; one thread per four
+// columns, every chunk requested before any is consumed.
+template <typename T>
+__global__ __launch_bounds__(256) void shrink_reduce_kernel(ShrinkArgs p) {
+  const int n_active = p.plan[H_NACTIVE];
+  const int quarter = p.rp >> 2;
+  const int64_t total = (int64_t)n_active * quarter;
+  const int32_t *__restrict__ perm = p.plan + p.off_perm;
+  const int32_t *__restrict__ prank = p.plan + p.off_prank;
+  const int64_t sstride = (int64_t)p.T * quarter;
+  const f32x4 *src = reinterpret_cast<const f32x4 *>(p.partial);
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (int64_t)gridDim.x * 256) {
+    const int pos = (int)(e / quarter), c4 = (int)(e - (int64_t)pos * quarter);
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
     for (int s0 = 0; s0 < p.ksplit; s0 += 8) {
-      unsigned long long q[8];
+      f32x4 q[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        q[u] = (s0 + u < p.ksplit)
-                   ? __hip_atomic_load(src + (s0 + u) * sstride + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                   : 0ull;
+      for (int u = 0; u < 8; ++u) q[u] = (s0 + u < p.ksplit) ? src[(s0 + u) * sstride + e] : f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const float2 f = __builtin_bit_cast(float2, q[u]);
-        v.x += f.x;
-        v.y += f.y;
-      }
+      for (int u = 0; u < 8; ++u) v += q[u];
     }
-    const int t = p.out_by_token ? perm[pos0 + row] : 0;
-    store_v<T>(p, pos0 + row, t, r, 2 * c2, v.x);
-    store_v<T>(p, pos0 + row, t, r, 2 * c2 + 1, v.y);
+    const int r = prank[pos];
+    const int t = p.out_by_token ? perm[pos] : 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) store_v<T>(p, pos, t, r, 4 * c4 + i, v[i]);
   }
-  if (tid == 0) p.counters[tile_idx] = 0;  // ready for the next launch that uses this plan
 }
 
 template <typename T, int MB, int NB>
@@ -123,7 +104,6 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs p) {
   using vec8 = typename Tr::vec8;
   constexpr int NBLK = MB * NB;
   __shared__ float red[2][NBLK * 256];
-  __shared__ int s_last;
 
   const int32_t *__restrict__ hdr = p.plan;
   const int tile_idx = blockIdx.x;
@@ -236,30 +216,33 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs p) {
         }
   }
   __syncthreads();
-  shrink_epilogue<T>(p, red[1], NB * 16, tile_idx, s, pos0, cnt, r, perm, &s_last);
+  shrink_epilogue<T>(p, red[1], NB * 16, s, pos0, cnt, r, perm);
 }
 
-// Prefill-sized tiles: GEMM structure.  The four waves split the tile's tokens (16*MBW each), so
-// no cross-wave reduction is needed; the adapter's A rows for the current 128-wide K step are
-// staged once per workgroup in LDS (double buffered) and shared by all waves, which cuts the
-// weight traffic into the compute unit by the tile height; x fragments still go straight from
-// global memory into MFMA registers.  The next step's A tile and x fragments are requested
-// before the current step is consumed.
-template <typename T, int MBW, int NB>
+// Prefill-sized tiles (128 tokens): GEMM structure with a three-stage LDS ring.
+//
+// The four waves split the tile's tokens (32 each), so no cross-wave reduction is needed.  Both
+// operands of a 64-wide K step go from global memory straight into LDS with 16-byte
+// global_load_lds (no registers are held while the data is in flight): every wave streams its
+// own x rows into a private part of the stage, the adapter's A rows are loaded once per
+// workgroup and shared by all waves.  A load instruction writes 1 KB to LDS in lane order, and
+// each lane asks for exactly the 16 bytes it will later feed to the matrix core, so the MFMA
+// operand read is ds_read_b128 at lane*16 -- conflict free, no layout conversion.  Two stages
+// are always in flight while the third is consumed; one s_barrier per K step.
+template <typename T, int NB>
 __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs p) {
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
-  constexpr int KC = (NB > 4) ? 64 : 128;     // K elements per step
-  constexpr int KS = KC / 32;                 // MFMA k-steps per step
-  constexpr int LDA = KC + 8;                 // LDS row stride (elements): 16 B of padding
-  constexpr int AV = NB * 16 * (KC / 8) / 256;  // 16-byte vectors of the A tile per thread
-  constexpr int VPR = KC / 8;                 // vectors per A row
-  // LDS: two A buffers during the K loop, then the workgroup's fp32 result tile
-  constexpr int A_BYTES = 2 * NB * 16 * LDA * 2;
-  constexpr int TILE_BYTES = 64 * MBW * NB * 16 * 4;
-  __shared__ __align__(16) unsigned char s_raw[A_BYTES > TILE_BYTES ? A_BYTES : TILE_BYTES];
-  uint16_t(*s_a)[NB * 16][LDA] = reinterpret_cast<uint16_t(*)[NB * 16][LDA]>(s_raw);
-  __shared__ int s_last;
+  constexpr int MBW = 2, KC = 64, KS = KC / 32, STAGES = 3;
+  constexpr int XBLK = MBW * KS;                        // 1 KB blocks of x per wave per stage
+  constexpr int ABLK = NB * KS;                         // 1 KB blocks of A per stage (shared)
+  constexpr int APW = ABLK >= 4 ? ABLK / 4 : 1;         // A blocks each wave loads per stage
+  constexpr int A_SLOTS = APW * 4;                      // >= ABLK; surplus slots hold duplicates
+  constexpr int STAGE_BYTES = (4 * XBLK + A_SLOTS) * 1024;
+  constexpr int TILE_BYTES = 128 * NB * 16 * 4;
+  constexpr int LOADS_PER_STAGE = XBLK + APW;           // per wave, identical for all waves
+  constexpr int RING_BYTES = STAGES * STAGE_BYTES + 1024;   // + one scratch block for dummy loads
+  __shared__ __align__(16) unsigned char s_raw[RING_BYTES > TILE_BYTES ? RING_BYTES : TILE_BYTES];
 
   const int32_t *__restrict__ hdr = p.plan;
   const int tile_idx = blockIdx.x;
@@ -272,9 +255,10 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs p) {
   const int lrow = lane & 15, kg = lane >> 4;
   const int32_t *__restrict__ perm = p.plan + p.off_perm;
   const int64_t base = (int64_t)astart + (int64_t)r * p.slot;
-  const int wrow0 = wave * 16 * MBW;          // first tile row of this wave
-  const bool wave_active = wrow0 < cnt;       // wave-uniform
+  const int wrow0 = wave * 16 * MBW;
+  const bool wave_active = wrow0 < cnt;                 // wave-uniform
 
+  // this lane's global row pointers
   const uint16_t *xp[MBW];
   bool xok[MBW];
 #pragma unroll
@@ -284,22 +268,64 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs p) {
     const int t = xok[mb] ? perm[pos0 + row] : 0;
     xp[mb] = p.x + (int64_t)t * p.h_in;
   }
-  // A staging role of this thread: vectors id = tid + i*256 -> (row = id / VPR, vector = id % VPR)
-  const uint16_t *ap[AV];
-  bool aok[AV];
-  int arow[AV], acv[AV];
+  // A blocks this wave loads: slot = wave*APW + i -> (nb, ks) = (slot / KS, slot % KS) when slot < ABLK
+  const uint16_t *ap[APW];
+  bool aok[APW];
+  int aks[APW];
 #pragma unroll
-  for (int i = 0; i < AV; ++i) {
-    const int id = tid + i * 256;
-    arow[i] = id / VPR;
-    acv[i] = id % VPR;
-    const int64_t idx = base + arow[i];
-    bool ok = arow[i] < r && idx >= 0 && idx < p.pool.a_loc_len;
+  for (int i = 0; i < APW; ++i) {
+    const int slot = (wave * APW + i) % ABLK;           // surplus slots duplicate real blocks
+    const int nb = slot / KS;
+    aks[i] = slot % KS;
+    const int j = nb * 16 + lrow;
+    const int64_t idx = base + j;
+    bool ok = j < r && idx >= 0 && idx < p.pool.a_loc_len;
     const int64_t prow = ok ? p.pool.a_loc[idx] : 0;
     ok = ok && prow >= 0 && prow < p.pool.w_rows;
     aok[i] = ok;
-    ap[i] = p.pool.w + (ok ? prow : 0) * p.h_in + acv[i] * 8;
+    ap[i] = p.pool.w + (ok ? prow : 0) * p.h_in;
   }
+
+  const int kbeg = s * p.kchunk;
+  const int kend = min(p.h_in, kbeg + p.kchunk);
+  const int n_steps = (kend - kbeg + KC - 1) / KC;
+
+  auto lds_x = [&](int stage, int blk) { return s_raw + stage * STAGE_BYTES + (wave * XBLK + blk) * 1024; };
+  auto lds_a = [&](int stage, int slot) { return s_raw + stage * STAGE_BYTES + (4 * XBLK + slot) * 1024; };
+  const u32x4 zero4 = {0, 0, 0, 0};
+
+  // Issue every load of one K step: EXACTLY LOADS_PER_STAGE load instructions per wave, because the
+  // consumer waits with a compile-time vmcnt.  A load whose lanes are all masked off would be skipped
+  // by the hardware branch around it, so in that case a dummy load into a scratch block is issued
+  // instead.  Lanes beyond the end of K write zeros into their own slot (no other lane touches it).
+  unsigned char *dummy = s_raw + STAGES * STAGE_BYTES;
+  auto load_or_dummy = [&](bool c, const uint16_t *src, unsigned char *dst) {
+    if (__builtin_amdgcn_ballot_w64(c) != 0ull) {
+      if (c) __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src), LDS_PTR(dst), 16, 0, 0);
+    } else {
+      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(p.plan), LDS_PTR(dummy), 16, 0, 0);
+    }
+  };
+  auto issue = [&](int step) {
+    const int stage = step % STAGES;
+    const int k0 = kbeg + step * KC;
+#pragma unroll
+    for (int mb = 0; mb < MBW; ++mb)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int k = k0 + ks * 32 + kg * 8;
+        unsigned char *dst = lds_x(stage, mb * KS + ks);
+        load_or_dummy(xok[mb] && k < kend, xp[mb] + k, dst);
+        if (k >= kend) lds_write16(lds_offset(dst) + lane * 16, zero4);
+      }
+#pragma unroll
+    for (int i = 0; i < APW; ++i) {
+      const int k = k0 + aks[i] * 32 + kg * 8;
+      unsigned char *dst = lds_a(stage, wave * APW + i);
+      load_or_dummy(aok[i] && k < kend, ap[i] + k, dst);
+      if (k >= kend) lds_write16(lds_offset(dst) + lane * 16, zero4);
+    }
+  };
 
   f32x4 acc[MBW][NB];
 #pragma unroll
@@ -307,66 +333,44 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs p) {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int kbeg = s * p.kchunk;
-  const int kend = min(p.h_in, kbeg + p.kchunk);
-
-  u32x4 xa[MBW][KS], na[AV];
-  auto load_x = [&](int k0, u32x4 (&dst)[MBW][KS]) {
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int k = k0 + ks * 32 + kg * 8;
-#pragma unroll
-      for (int mb = 0; mb < MBW; ++mb) dst[mb][ks] = (xok[mb] && k < kend) ? load16(xp[mb] + k) : u32x4{0, 0, 0, 0};
-    }
-  };
-  auto load_a = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < AV; ++i) na[i] = (aok[i] && k0 + acv[i] * 8 < kend) ? load16(ap[i] + k0) : u32x4{0, 0, 0, 0};
-  };
-  auto store_a = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < AV; ++i) *reinterpret_cast<u32x4 *>(&s_a[buf][arow[i]][acv[i] * 8]) = na[i];
-  };
-
-  load_a(kbeg);
-  load_x(kbeg, xa);
-  store_a(0);
-  __syncthreads();
-  int buf = 0;
-  for (int k0 = kbeg; k0 < kend; k0 += KC) {
-    const bool more = k0 + KC < kend;  // workgroup-uniform
-    u32x4 nx[MBW][KS];
-    if (more) {
-      load_a(k0 + KC);
-      load_x(k0 + KC, nx);
-    }
+  issue(0);
+  if (n_steps > 1) issue(1);
+  for (int step = 0; step < n_steps; ++step) {
+    // wait for this step's loads (the next step's may stay in flight), then meet the other waves:
+    // after the barrier the stage is complete for everybody and the stage consumed in the previous
+    // iteration is free to be refilled
+    if (step + 1 < n_steps) wait_vmcnt<LOADS_PER_STAGE>(); else wait_vmcnt<0>();
+    wait_lgkmcnt0();
+    __builtin_amdgcn_s_barrier();
+    if (step + 2 < n_steps) issue(step + 2);
+    const int stage = step % STAGES;
     if (wave_active) {
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
+        u32x4 xf[MBW], bf[NB];
+#pragma unroll
+        for (int mb = 0; mb < MBW; ++mb) xf[mb] = lds_read16(lds_offset(lds_x(stage, mb * KS + ks)) + lane * 16);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) bf[nb] = lds_read16(lds_offset(lds_a(stage, nb * KS + ks)) + lane * 16);
+        wait_lgkmcnt0();
+#pragma unroll
+        for (int mb = 0; mb < MBW; ++mb) pin(xf[mb]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) pin(bf[nb]);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           if (nb * 16 < r) {
-            const u32x4 bf = *reinterpret_cast<const u32x4 *>(&s_a[buf][nb * 16 + lrow][ks * 32 + kg * 8]);
 #pragma unroll
             for (int mb = 0; mb < MBW; ++mb)
-              acc[mb][nb] = Tr::mfma(as<vec8>(xa[mb][ks]), as<vec8>(bf), acc[mb][nb]);
+              acc[mb][nb] = Tr::mfma(as<vec8>(xf[mb]), as<vec8>(bf[nb]), acc[mb][nb]);
           }
         }
       }
     }
-    if (more) {
-      store_a(buf ^ 1);
-#pragma unroll
-      for (int mb = 0; mb < MBW; ++mb)
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) xa[mb][ks] = nx[mb][ks];
-    }
-    __syncthreads();
-    buf ^= 1;
   }
+  wait_lgkmcnt0();
+  __syncthreads();   // everybody is done reading the ring: reuse it for the result tile
 
-  // every wave holds the complete K-chunk sums of its own tokens: lay the tile out row-major
-  // in LDS (the A buffers are free after the loop's last barrier)
   float *otile = reinterpret_cast<float *>(s_raw);
 #pragma unroll
   for (int mb = 0; mb < MBW; ++mb)
@@ -379,16 +383,16 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs p) {
         otile[row * (NB * 16) + col] = acc[mb][nb][i];
       }
   __syncthreads();
-  shrink_epilogue<T>(p, otile, NB * 16, tile_idx, s, pos0, cnt, r, perm, &s_last);
+  shrink_epilogue<T>(p, otile, NB * 16, s, pos0, cnt, r, perm);
 }
 
-template <typename T, int MBW>
+template <typename T>
 int launch_gemm_nb(hipStream_t st, const ShrinkArgs &a, int nb, dim3 grid) {
   switch (nb) {
-    case 1: hipLaunchKernelGGL((shrink_gemm_kernel<T, MBW, 1>), grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((shrink_gemm_kernel<T, MBW, 2>), grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL((shrink_gemm_kernel<T, MBW, 4>), grid, dim3(256), 0, st, a); break;
-    case 8: hipLaunchKernelGGL((shrink_gemm_kernel<T, MBW, 8>), grid, dim3(256), 0, st, a); break;
+    case 1: hipLaunchKernelGGL((shrink_gemm_kernel<T, 1>), grid, dim3(256), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((shrink_gemm_kernel<T, 2>), grid, dim3(256), 0, st, a); break;
+    case 4: hipLaunchKernelGGL((shrink_gemm_kernel<T, 4>), grid, dim3(256), 0, st, a); break;
+    case 8: hipLaunchKernelGGL((shrink_gemm_kernel<T, 8>), grid, dim3(256), 0, st, a); break;
     default: return fail(MLORA_ERR_NO_KERNEL, "shrink: no kernel for rank blocks=%d", nb);
   }
   return check_launch("shrink_gemm_kernel");
@@ -412,12 +416,24 @@ int launch_shrink_t(hipStream_t st, const ShrinkArgs &a, int bm, int nb, dim3 gr
     case 16: return launch_shrink_nb<T, 1>(st, a, nb, grid);
     case 32: return launch_shrink_nb<T, 2>(st, a, nb, grid);
     case 64: return launch_shrink_nb<T, 4>(st, a, nb, grid);
-    case 128: return launch_gemm_nb<T, 2>(st, a, nb, grid);
+    case 128: return launch_gemm_nb<T>(st, a, nb, grid);
     default: return fail(MLORA_ERR_NO_KERNEL, "shrink: tile height %d not in {16,32,64,128}", bm);
   }
 }
 
 }  // namespace
+
+int launch_shrink_reduce(hipStream_t st, const ShrinkArgs &a, mlora_dtype dt) {
+  if (a.T <= 0) return MLORA_OK;
+  int64_t blocks = ((int64_t)a.T * (a.rp >> 2) + 255) / 256;
+  if (blocks > 2048) blocks = 2048;
+  if (blocks < 1) blocks = 1;
+  if (dt == MLORA_F16)
+    hipLaunchKernelGGL(shrink_reduce_kernel<_Float16>, dim3((unsigned)blocks), dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL(shrink_reduce_kernel<__bf16>, dim3((unsigned)blocks), dim3(256), 0, st, a);
+  return check_launch("shrink_reduce_kernel");
+}
 
 int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int64_t grid_tiles,
                   mlora_dtype dt) {
