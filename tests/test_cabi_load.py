@@ -88,7 +88,9 @@ def test_missing_library_fails_loudly(monkeypatch):
 def test_tile_table_lookup_and_fallback():
     from valora_amd import tile_table as tt
     cfg = tt.lookup(256, 16, 4096, 64)
-    assert cfg.bm_shrink in (16, 32, 64) and 1 <= cfg.ksplit <= 64 and cfg.bm_expand % 16 == 0
-    fb = tt.fallback(100000, 128, 4096, 4)
-    assert fb.bm_shrink <= 32 and fb.ksplit >= 1
+    assert cfg.bm_shrink in (16, 32, 64, 128) and 1 <= cfg.ksplit <= 64 and cfg.bm_expand % 16 == 0
+    fb = tt.fallback(100000, 128, 4096, 4)          # long runs per adapter -> LDS-staged 128-token tiles
+    assert fb.bm_shrink == 128 and fb.ksplit >= 1 and not fb.reduce_in_expand
+    fb = tt.fallback(300, 64, 4096, 200)            # decode-like -> direct 16-token tiles, expand sums the chunks
+    assert fb.bm_shrink == 16 and fb.reduce_in_expand
     assert tt.key(300, 16, 4096, 64) == "1024:16:4096:128"

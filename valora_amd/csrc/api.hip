@@ -74,20 +74,23 @@ int check_dims(int64_t T, int64_t wide, int64_t narrow, int64_t h_in, int64_t h_
   return MLORA_OK;
 }
 
+// defaults measured on MI355X (see valora_amd/tile_table.json for the per-shape table the Python
+// host layer uses): 128-token LDS-staged tiles once adapters own long runs of tokens
 int default_bm_shrink(int64_t T, int64_t A) {
-  (void)A;
-  return T <= 2048 ? 16 : T <= 8192 ? 32 : 64;
+  const int64_t groups = A < T ? (A > 0 ? A : 1) : (T > 0 ? T : 1);
+  if (T > 4096 && T / groups >= 64) return 128;
+  return T <= 1024 ? 16 : 32;
 }
 int default_bm_expand(int64_t T, int64_t A) {
   (void)A;
-  return T <= 1024 ? 32 : T <= 8192 ? 64 : 128;
+  return T <= 1024 ? 16 : T <= 4096 ? 32 : 128;
 }
 int default_ksplit(int64_t T, int64_t A, int bm, int64_t h_in) {
   // aim for >= ~1024 workgroups, keep >= 256 K elements per workgroup, at most 16 partials
   int64_t tiles = tiles_upper(T, A, bm);
   if (tiles > T) tiles = T;
   if (tiles < 1) tiles = 1;
-  int64_t ks = (1024 + tiles - 1) / tiles;
+  int64_t ks = (768 + tiles - 1) / tiles;
   int64_t kmax = h_in / 256;
   if (kmax < 1) kmax = 1;
   if (ks > kmax) ks = kmax;

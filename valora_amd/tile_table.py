@@ -43,12 +43,14 @@ def key(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> str:
 
 
 def fallback(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> TileConfig:
-    bm_s = 16 if n_tokens <= 2048 else 32 if n_tokens <= 8192 else 64
-    if max_rank > 64:
-        bm_s = min(bm_s, 32)
+    tokens_per_adapter = n_tokens / max(1, min(n_adapters, n_tokens))
+    if n_tokens > 4096 and tokens_per_adapter >= 64:
+        bm_s = 128
+    else:
+        bm_s = 16 if n_tokens <= 1024 else 32
     tiles = max(1, min(n_tokens, -(-n_tokens // bm_s) + min(n_adapters, n_tokens)))
-    ksplit = max(1, min(16, hidden // 256, -(-1024 // tiles)))
-    bm_e = 32 if n_tokens <= 1024 else 64 if n_tokens <= 8192 else 128
+    ksplit = max(1, min(16, hidden // 256, -(-768 // tiles)))
+    bm_e = 16 if n_tokens <= 1024 else 32 if n_tokens <= 4096 else 128
     return TileConfig(bm_s, ksplit, bm_e, n_tokens <= 1024)
 
 
