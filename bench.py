@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # scaled by the same counters' reading for a plain copy of known size; None until measured.
-MEASURED_TRAFFIC_BYTES = None
+MEASURED_TRAFFIC_BYTES = {"expand_kernel": 13_030_000, "shrink_kernel": 10_520_000}  # profiles/config2_decode_hbm_traffic_pmc.txt
 
 
 def parse():
@@ -44,6 +44,9 @@ def parse():
     ap.add_argument("--reduce-in-expand", type=int, default=None, help="1: expand sums the split-K chunks, 0: shrink does")
     ap.add_argument("--fused", action="store_true", help="use the single-launch fused kernel instead of shrink + expand")
     ap.add_argument("--replicas", type=int, default=0, help="output slices per tile of the fused kernel (0 = default)")
+    ap.add_argument("--pmc-copy-mib", type=int, default=0,
+                    help="first run one plain device copy of this many MiB: a kernel of known traffic to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings with")
     ap.add_argument("--all-configs", metavar="FILE", default=None,
                     help="also measure every target of configs 1,3,4,5 and write a JSON report to FILE")
     return ap.parse_args()
@@ -198,6 +201,13 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
+    if args.pmc_copy_mib > 0:
+        src = torch.ones(args.pmc_copy_mib << 19, dtype=torch.float16, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)          # reads and writes exactly pmc_copy_mib MiB
+        torch.cuda.synchronize()
+        del src, dst
     L = args.layers
     w, wd, kb, vb, xs, ys = build_layers(torch, W, dev, L)
     t = wd.targets[0]
@@ -270,7 +280,7 @@ def main():
         dom = ("expand_kernel", bytes_expand, ex_us) if ex_us >= sh_us else ("shrink_kernel", bytes_shrink, sh_us)
     achieved = dom[1] / (dom[2] * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(dom[0]),
                 "kernel": dom[0], "algorithmic_bytes_per_launch": dom[1], "avg_launch_us": round(dom[2], 3),
                 "shrink_kernel_us": round(sh_us, 3), "expand_kernel_us": round(ex_us, 3),
                 "op_bytes": bytes_op, "op_us_events": round(op_us, 3),
