@@ -23,6 +23,7 @@ namespace {
 constexpr int EXP_BN = 256;       // outputs per workgroup
 constexpr int EXP_WN = 64;        // outputs per wave
 constexpr int STAGE_LD = EXP_WN + 4;
+constexpr int EXP_MBU = 2;         // 16-token blocks whose loads are in flight together
 constexpr int EXP_MAX_BM = 256;   // tallest expand tile (tokens), one thread per token at set-up
 
 template <typename T, int KB, bool PARTIAL>
@@ -91,84 +92,95 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
   const int rr0 = lane >> 3, c8 = (lane & 7) * 8;
   const bool ocol_ok = (o_wave + c8) < p.h_out;
 
+  // Two 16-token blocks per iteration: their y rows and v fragments are all requested before either
+  // block is consumed, so an iteration costs one memory round trip for 32 tokens.
   const int n_mb = (cnt + 15) >> 4;
-  for (int mb = 0; mb < n_mb; ++mb) {
-    // ---- y rows first (the longest-latency loads of the iteration)
-    u32x4 yv[2];
-    uint16_t *yp[2];
-    bool yok[2];
+  for (int mb0 = 0; mb0 < n_mb; mb0 += EXP_MBU) {
+    u32x4 yv[EXP_MBU][2];
+    uint16_t *yp[EXP_MBU][2];
+    bool yok[EXP_MBU][2];
+    u32x4 vfrag[EXP_MBU][KB];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int row = mb * 16 + rr0 + 8 * h;
-      yok[h] = ocol_ok && row < cnt;
-      const int t = yok[h] ? s_perm[row] : 0;
-      yp[h] = p.y + (int64_t)t * p.h_out + o_wave + c8;
-      yv[h] = yok[h] ? load16(yp[h]) : u32x4{0, 0, 0, 0};
-    }
-    // ---- v fragments: rows = tokens (lrow), 8 consecutive rank elements per lane
-    const int prow = mb * 16 + lrow;
-    const bool pok = prow < cnt;
-    u32x4 vfrag[KB];
+    for (int b = 0; b < EXP_MBU; ++b) {
+      const int mb = mb0 + b;
+      // ---- y rows first (the longest-latency loads of the iteration)
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb) {
-      const int j0 = kb * 32 + kg * 8;
-      u32x4 v = {0, 0, 0, 0};
-      if (pok && j0 < rk) {
-        if constexpr (PARTIAL) {
-          // split-K partials of the shrink: all chunks are requested before any is consumed,
-          // summed in chunk order and rounded to T once
-          float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          const float *src0 = p.partial + ((int64_t)pos0 + prow) * p.rp + j0;
-          const int64_t sstride = (int64_t)p.T * p.rp;
-          for (int s0 = 0; s0 < p.ksplit; s0 += 4) {
-            f32x4 lo[4], hi[4];
+      for (int h = 0; h < 2; ++h) {
+        const int row = mb * 16 + rr0 + 8 * h;
+        yok[b][h] = ocol_ok && row < cnt;
+        const int t = yok[b][h] ? s_perm[row] : 0;
+        yp[b][h] = p.y + (int64_t)t * p.h_out + o_wave + c8;
+        yv[b][h] = yok[b][h] ? load16(yp[b][h]) : u32x4{0, 0, 0, 0};
+      }
+      // ---- v fragments: rows = tokens (lrow), 8 consecutive rank elements per lane
+      const int prow = mb * 16 + lrow;
+      const bool pok = prow < cnt;
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-              const bool ok = s0 + u < p.ksplit;
-              const f32x4 *src = reinterpret_cast<const f32x4 *>(src0 + (int64_t)(s0 + u) * sstride);
-              lo[u] = ok ? src[0] : f32x4{0.f, 0.f, 0.f, 0.f};
-              hi[u] = ok ? src[1] : f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int kb = 0; kb < KB; ++kb) {
+        const int j0 = kb * 32 + kg * 8;
+        u32x4 v = {0, 0, 0, 0};
+        if (pok && j0 < rk) {
+          if constexpr (PARTIAL) {
+            // split-K partials of the shrink: all chunks are requested before any is consumed,
+            // summed in chunk order and rounded to T once
+            float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            const float *src0 = p.partial + ((int64_t)pos0 + prow) * p.rp + j0;
+            const int64_t sstride = (int64_t)p.T * p.rp;
+            for (int s0 = 0; s0 < p.ksplit; s0 += 4) {
+              f32x4 lo[4], hi[4];
+#pragma unroll
+              for (int u = 0; u < 4; ++u) {
+                const bool ok = s0 + u < p.ksplit;
+                const f32x4 *src = reinterpret_cast<const f32x4 *>(src0 + (int64_t)(s0 + u) * sstride);
+                lo[u] = ok ? src[0] : f32x4{0.f, 0.f, 0.f, 0.f};
+                hi[u] = ok ? src[1] : f32x4{0.f, 0.f, 0.f, 0.f};
+              }
+#pragma unroll
+              for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { f[i] += lo[u][i]; f[4 + i] += hi[u][i]; }
             }
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-#pragma unroll
-              for (int i = 0; i < 4; ++i) { f[i] += lo[u][i]; f[4 + i] += hi[u][i]; }
+            v = pack8<T>(f);
+          } else {
+            const int64_t vrow = p.v_by_pos ? (int64_t)(pos0 + prow) : (int64_t)s_perm[prow];
+            v = load16(p.v + vrow * p.v_stride + j0);
           }
-          v = pack8<T>(f);
-        } else {
-          const int64_t vrow = p.v_by_pos ? (int64_t)(pos0 + prow) : (int64_t)s_perm[prow];
-          v = load16(p.v + vrow * p.v_stride + j0);
         }
-      }
-      vfrag[kb] = v;
-    }
-    // ---- delta block through the matrix cores, staged to LDS in token-major order
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb)
-        if (kb * 32 < rk) acc = Tr::mfma(as<vec8>(vfrag[kb]), as<vec8>(bfrag[nb][kb]), acc);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) stage[wave][kg * 4 + i][nb * 16 + lrow] = acc[i];
-    }
-    // stage[wave] is private to this wave and a wave's LDS operations execute in order, so only
-    // the compiler has to be kept from reordering the reads below over the writes above.
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      if (yok[h]) {
-        const float *srow = &stage[wave][rr0 + 8 * h][c8];
-        float f[8];
-        unpack8<T>(yv[h], f);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f[i] += scale * srow[i];
-        store16(yp[h], pack8<T>(f));
+        vfrag[b][kb] = v;
       }
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int b = 0; b < EXP_MBU; ++b) {
+      if (mb0 + b < n_mb) {   // workgroup-uniform
+        // ---- delta block through the matrix cores, staged to LDS in token-major order
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+          f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb)
+            if (kb * 32 < rk) acc = Tr::mfma(as<vec8>(vfrag[b][kb]), as<vec8>(bfrag[nb][kb]), acc);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) stage[wave][kg * 4 + i][nb * 16 + lrow] = acc[i];
+        }
+        // stage[wave] is private to this wave and a wave's LDS operations execute in order, so only
+        // the compiler has to be kept from reordering the reads below over the writes above.
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          if (yok[b][h]) {
+            const float *srow = &stage[wave][rr0 + 8 * h][c8];
+            float f[8];
+            unpack8<T>(yv[b][h], f);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f[i] += scale * srow[i];
+            store16(yp[b][h], pack8<T>(f));
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+      }
+    }
   }
 }
 
