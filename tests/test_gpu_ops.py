@@ -191,3 +191,55 @@ def test_sgmm_and_prefill_entry_points(dev, dtype):
         want = O.triton_expand(v, pool.value_buffer.view(-1, h), y0, pool.a_scaling, pool.a_loc, pool.a_start,
                                pool.a_len, start, seq, req, h, 2, R, mx)
         assert_parity(y.cpu(), want, f"prefill expand mx={mx}")
+
+
+def test_edge_cases_empty_and_no_adapter(dev):
+    """T = 0, a batch where no token has an adapter, one token, and pools with 1 or 2 slots."""
+    from valora_amd.kernels import dispatch_bgmv
+    from valora_amd.plan import LoraPlan
+    dtype = torch.float16
+    pool, ids, x, y0, v, R = _case(31, 20, 512, 512, (8, 16), dtype)
+    pd = pool.to(dev)
+    idx = (pd.a_start, pd.a_len, pd.a_loc)
+    # T = 0: nothing happens, nothing is read
+    e = torch.zeros(0, 512, dtype=dtype, device=dev)
+    d = torch.zeros(0, 16, dtype=dtype, device=dev)
+    dispatch_bgmv(d, e, pd.key_buffer, *idx, torch.zeros(0, dtype=torch.long, device=dev), 0, pd.a_scaling)
+    dispatch_bgmv(e, d, pd.value_buffer, *idx, torch.zeros(0, dtype=torch.long, device=dev), 0, pd.a_scaling)
+    plan = LoraPlan(torch.zeros(0, dtype=torch.long, device=dev), pd.a_start, pd.a_len, 16, hidden=512)
+    plan.apply(e, e.clone(), pd.key_buffer, pd.value_buffer, *idx, 0, pd.a_scaling)
+    assert plan.header()["n_active"] == 0
+    # no token has an adapter: y comes back bit-identical
+    none = torch.full((20,), -1, dtype=torch.long, device=dev)
+    y = y0.to(dev)
+    plan = LoraPlan(none, pd.a_start, pd.a_len, 16, hidden=512)
+    plan.apply(y, x.to(dev), pd.key_buffer, pd.value_buffer, *idx, 1, pd.a_scaling)
+    assert torch.equal(y.cpu(), y0)
+    # one token
+    y = y0[:1].to(dev)
+    plan = LoraPlan(ids[:1].to(dev), pd.a_start, pd.a_len, 16, hidden=512)
+    plan.apply(y, x[:1].to(dev), pd.key_buffer, pd.value_buffer, *idx, 2, pd.a_scaling)
+    want = O.lora_op(y0[:1], x[:1], pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc,
+                     ids[:1], 2, pool.a_scaling)
+    assert_parity(y.cpu(), want, "one token")
+    # pools with other slot counts (a_len = n_slots * r)
+    for n_slots in (1, 2, 7):
+        g = torch.Generator().manual_seed(n_slots)
+        p2 = W.make_pool([8, 32, 16], 256, 384, dtype, g, True, n_slots=n_slots, std=0.05, heads=8)
+        ids2 = torch.randint(0, 3, (50,), generator=g)
+        x2 = torch.randn(50, 256, generator=g).to(dtype)
+        y2 = torch.randn(50, 384, generator=g).to(dtype)
+        p2d = p2.to(dev)
+        slot = n_slots - 1
+        plan = LoraPlan(ids2.to(dev), p2d.a_start, p2d.a_len, 32, n_slots=n_slots, hidden=256)
+        yy = y2.to(dev)
+        plan.apply(yy, x2.to(dev), p2d.key_buffer, p2d.value_buffer, p2d.a_start, p2d.a_len, p2d.a_loc, slot,
+                   p2d.a_scaling)
+        want = O.lora_op(y2, x2, p2.key_buffer, p2.value_buffer, p2.a_start, p2.a_len, p2.a_loc, ids2, slot,
+                         p2.a_scaling, n_slots=n_slots)
+        assert_parity(yy.cpu(), want, f"n_slots={n_slots}")
+        yy = y2.to(dev)
+        plan16 = LoraPlan(ids2.to(dev), p2d.a_start, p2d.a_len, 32, n_slots=n_slots, hidden=256, bm_shrink=16)
+        plan16.apply_fused(yy, x2.to(dev), p2d.key_buffer, p2d.value_buffer, p2d.a_start, p2d.a_len, p2d.a_loc, slot,
+                           p2d.a_scaling)
+        assert_parity(yy.cpu(), want, f"fused n_slots={n_slots}")
