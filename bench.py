@@ -179,8 +179,34 @@ def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph):
                             "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4), "tflops": round(f / us / 1e6, 2),
                             "tile": [plan.bm_shrink, plan.ksplit, plan.bm_expand]}
             total_us += us
+        # targets that read the same x, in one shrink + one expand launch
+        groups, fused_total = {}, total_us
+        for names in (("q", "k", "v"), ("gate", "up")):
+            ts = [t for t in wd.targets if t.name in names]
+            if len(ts) < 2:
+                continue
+            p = ts[0].pool
+            plan = LoraPlan(wd.ids, p.a_start, p.a_len, R, hidden=ts[0].h_in)
+            ycopies = [[wd.y0[t.name].clone() for t in ts] for _ in range(4)]
+            x, slots = wd.x[ts[0].h_in], [t.slot for t in ts]
+
+            def fm():
+                for ys in ycopies:
+                    plan.apply_multi(ys, x, p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, slots,
+                                     p.a_scaling)
+
+            ms, _ = time_graph(torch, fm, 30, 3, use_graph)
+            us = ms * 1e3 / 4
+            separate = sum(rows[t.name]["us"] for t in ts)
+            # x is read once for the whole group
+            b = sum(w.algorithmic_bytes(t.name) for t in ts) - (len(ts) - 1) * w.T * ts[0].h_in * 2
+            groups["+".join(t.name for t in ts)] = {"us": round(us, 2), "separate_us": round(separate, 2),
+                                                    "bytes": b, "gbps": round(b / us / 1e3, 1),
+                                                    "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            fused_total += us - separate
         report[f"config{n}"] = {"tokens": w.T, "dtype": str(w.dtype), "max_rank": R, "targets": rows,
-                                "us_per_layer": round(total_us, 2)}
+                                "us_per_layer": round(total_us, 2), "multi_target": groups,
+                                "us_per_layer_multi_target": round(fused_total, 2)}
         del wd
         torch.cuda.empty_cache()
     with open(path, "w") as f:

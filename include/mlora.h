@@ -20,6 +20,8 @@ extern "C" {
 
 typedef enum { MLORA_F16 = 0, MLORA_BF16 = 1 } mlora_dtype;
 
+#define MLORA_MAX_TARGETS 4   /* targets one mlora_lora_apply_multi call can take */
+
 typedef enum {
   MLORA_OK = 0,
   MLORA_ERR_INVALID = -1,     /* bad argument (null pointer, negative size, misaligned base) */
@@ -143,6 +145,26 @@ int mlora_lora_apply(void *stream, const mlora_plan *plan, void *scratch, size_t
                      int64_t max_rank, const mlora_pool *pool_a, const mlora_pool *pool_b,
                      int32_t slot, const void *scales, int32_t ksplit, int32_t flags,
                      mlora_dtype dtype);
+
+/* One output of a multi-target call: y += scale * v_slot * B_slot. */
+typedef struct {
+  void *y;                  /* [T, h_out], updated in place                                      */
+  const void *w_b;          /* value buffer holding this target's B rows (row width h_out)        */
+  int64_t w_b_rows;
+  int32_t slot;             /* slot of the adapter index this target uses (A rows and B rows)     */
+} mlora_target;
+
+/* Shrink + expand for several targets that read the same x (q, k, v of one layer; gate and up):
+ * one shrink launch for all targets, one expand launch for all targets.  The targets share h_in,
+ * h_out, the key buffer and the adapter index of pool_a; each has its own y, value buffer and slot.
+ * Replaces the reference's 3 + 3 launches per attention block
+ * (valora/models/peft/lora_unordered_batch_infer.py:946-988).  scratch_bytes must be at least
+ * n_targets * mlora_scratch_bytes(T, max_rank, ksplit).  Results are identical to n_targets
+ * separate mlora_lora_apply calls.                                                              */
+int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, size_t scratch_bytes,
+                           const void *x, int64_t T, int64_t h_in, int64_t h_out, int64_t max_rank,
+                           const mlora_pool *pool_a, int32_t n_targets, const mlora_target *targets,
+                           const void *scales, int32_t ksplit, int32_t flags, mlora_dtype dtype);
 
 /* Shrink + expand of one target in ONE launch, for decode-like batches (few tokens per adapter):
  * each workgroup recomputes v for its tile of <= 16 tokens and expands one slice of the output

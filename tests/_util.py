@@ -44,6 +44,18 @@ def run_plan(wd, name, **kw):
     return y
 
 
+def run_multi(wd, names, **kw):
+    """Targets that read the same x and live in the same pool, through LoraPlan.apply_multi."""
+    from valora_amd.plan import LoraPlan
+    ts = [wd.target(n) for n in names]
+    p = ts[0].pool
+    plan = LoraPlan(wd.ids, p.a_start, p.a_len, max_rank(wd), hidden=ts[0].h_in, **kw)
+    ys = [wd.y0[n].clone() for n in names]
+    plan.apply_multi(ys, wd.x[ts[0].h_in], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc,
+                     [t.slot for t in ts], p.a_scaling)
+    return ys
+
+
 def run_fused(wd, name, replicas=0):
     from valora_amd.plan import LoraPlan
     t = wd.target(name); p = t.pool

@@ -9,8 +9,8 @@ import torch
 
 from oracle import lora_oracle as O
 from valora_amd import workloads as W
-from tests._util import (assert_parity, max_rank, oracle_target, run_bgmv, run_fused, run_plan, run_prefill,
-                         run_sgmm)
+from tests._util import (assert_parity, max_rank, oracle_target, run_bgmv, run_fused, run_multi, run_plan,
+                         run_prefill, run_sgmm)
 
 pytestmark = pytest.mark.gpu
 
@@ -43,6 +43,28 @@ def test_small_configs_all_entry_points(dev, n):
             assert_parity(y.cpu(), want, f"config{n}/{t.name}/bgmv")
             assert_parity(run_sgmm(wd, t.name).cpu(), want, f"config{n}/{t.name}/sgmm")
             assert_parity(run_prefill(wd, t.name).cpu(), want, f"config{n}/{t.name}/prefill")
+
+
+MULTI_GROUPS = {1: [("q",)], 2: [("q",)], 3: [("q", "k", "v"), ("gate", "up"), ("o",)],
+                4: [("q", "k", "v"), ("gate", "up")], 5: [("q", "k", "v"), ("gate", "up"), ("down",)]}
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5])
+def test_small_configs_multi_target(dev, n):
+    """Targets that share x in one shrink + one expand launch: bit-identical to one call per target."""
+    w = W.CONFIGS[n](**SMALL[n])
+    wd = w.to(dev)
+    have = {t.name for t in w.targets}
+    for names in MULTI_GROUPS[n]:
+        names = tuple(x for x in names if x in have)
+        if not names:
+            continue
+        for kw in (dict(), dict(ksplit=4, reduce_in_expand=False), dict(ksplit=4, reduce_in_expand=True),
+                   dict(ksplit=1, bm_shrink=128, bm_expand=64)):
+            ys = run_multi(wd, names, **kw)
+            for name, y in zip(names, ys):
+                assert_parity(y.cpu(), oracle_target(w, name), f"config{n}/{name}/multi {kw}")
+                assert torch.equal(y, run_plan(wd, name, **kw)), f"config{n}/{name}: multi differs from single {kw}"
 
 
 def test_config1_full_vs_per_segment_reference(dev):
@@ -105,6 +127,16 @@ def test_full_configs_gemm_shrink_tiles(dev, n, name):
         for rie in (False, True):
             assert_parity(run_plan(wd, name, bm_shrink=128, ksplit=ks, bm_expand=128, reduce_in_expand=rie).cpu(), want,
                           f"config{n}/{name}/plan bm=128 ks={ks} reduce_in_expand={rie}")
+
+
+@pytest.mark.parametrize("n,names", [(3, ("q", "k", "v")), (4, ("gate", "up")), (5, ("q", "k", "v"))])
+def test_full_configs_multi_target(dev, n, names):
+    w = W.CONFIGS[n]()
+    wd = w.to(dev)
+    ys = run_multi(wd, names)
+    for name, y in zip(names, ys):
+        assert torch.equal(y, run_plan(wd, name)), f"config{n}/{name}: multi differs from single"
+    assert_parity(ys[0].cpu(), oracle_target(w, names[0]), f"config{n}/{names[0]}/multi")
 
 
 def test_rank128_both_shrink_kernels(dev):

@@ -24,7 +24,7 @@ SYMBOLS = [
     "mlora_last_error", "mlora_version", "mlora_plan_bytes", "mlora_scratch_bytes",
     "mlora_workspace_bytes", "mlora_build_plan", "mlora_count_consecutive",
     "mlora_ids_from_segments", "mlora_ids_from_requests", "mlora_shrink", "mlora_expand", "mlora_lora_apply",
-    "mlora_lora_fused", "mlora_dispatch_bgmv",
+    "mlora_lora_apply_multi", "mlora_lora_fused", "mlora_dispatch_bgmv",
     "mlora_dispatch_sgmm", "mlora_prefill_shrink", "mlora_prefill_expand",
 ]
 
@@ -33,6 +33,13 @@ class Pool(ctypes.Structure):
     _fields_ = [("w", c_void_p), ("w_rows", c_int64), ("a_start", c_void_p), ("a_len", c_void_p),
                 ("a_loc", c_void_p), ("n_adapters", c_int64), ("a_loc_len", c_int64),
                 ("n_slots", c_int32)]
+
+
+class Target(ctypes.Structure):
+    _fields_ = [("y", c_void_p), ("w_b", c_void_p), ("w_b_rows", c_int64), ("slot", c_int32)]
+
+
+MAX_TARGETS = 4
 
 
 class Plan(ctypes.Structure):
@@ -74,6 +81,9 @@ def lib():
     L.mlora_lora_apply.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_size_t, c_void_p, c_void_p,
                                    c_int64, c_int64, c_int64, c_int64, POINTER(Pool), POINTER(Pool),
                                    c_int32, c_void_p, c_int32, c_int32, c_int]
+    L.mlora_lora_apply_multi.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_size_t, c_void_p, c_int64, c_int64,
+                                         c_int64, c_int64, POINTER(Pool), c_int32, POINTER(Target), c_void_p,
+                                         c_int32, c_int32, c_int]
     L.mlora_lora_fused.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                    POINTER(Pool), POINTER(Pool), c_int32, c_void_p, c_int32, c_int]
     L.mlora_dispatch_bgmv.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,

@@ -254,6 +254,10 @@ int mlora_shrink(void *stream, const mlora_plan *plan, void *scratch, size_t scr
   a.ksplit = ksplit;
   a.kchunk = (int)align_up((h_in + ksplit - 1) / ksplit, 128);
   a.partial_only = (!out && ksplit > 1 && (flags & MLORA_REDUCE_IN_EXPAND)) ? 1 : 0;
+  a.n_targets = 1;
+  for (int i = 0; i < MLORA_MAX_TARGETS; ++i) a.slots[i] = slot;
+  a.out_tstride = 0;
+  a.partial_tstride = 0;
   if (out) {
     a.out = static_cast<uint16_t *>(out);
     a.out_stride = out_stride;
@@ -316,6 +320,15 @@ int mlora_expand(void *stream, const mlora_plan *plan, void *y, int64_t T, int64
   a.kmax = (int)max_rank;
   a.slot = slot;
   a.n_ochunks = (int)((h_out + expand_bn() - 1) / expand_bn());
+  a.n_targets = 1;
+  for (int i = 0; i < MLORA_MAX_TARGETS; ++i) {
+    a.slots[i] = slot;
+    a.ys[i] = a.y;
+    a.ws[i] = a.pool.w;
+    a.w_rows_t[i] = a.pool.w_rows;
+  }
+  a.v_tstride = 0;
+  a.partial_tstride = 0;
   return launch_expand((hipStream_t)stream, a, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand),
                        dtype);
 }
@@ -331,6 +344,100 @@ int mlora_lora_apply(void *stream, const mlora_plan *plan, void *scratch, size_t
     return rc;
   return mlora_expand(stream, plan, y, T, h_out, scratch, nullptr, 0, max_rank, pool_b, slot, scales, ksplit, flags,
                       dtype);
+}
+
+int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, size_t scratch_nbytes, const void *x,
+                           int64_t T, int64_t h_in, int64_t h_out, int64_t max_rank, const mlora_pool *pool_a,
+                           int32_t n_targets, const mlora_target *targets, const void *scales, int32_t ksplit,
+                           int32_t flags, mlora_dtype dtype) {
+  if (int rc = check_dtype(dtype, h_in, h_out)) return rc;
+  if (int rc = check_dims(T, h_in, max_rank, h_in, h_out, dtype)) return rc;
+  if (int rc = check_dims(T, h_out, max_rank, h_in, h_out, dtype)) return rc;
+  if (int rc = check_plan(plan, T, "lora_apply_multi")) return rc;
+  if (int rc = check_pool(pool_a, "lora_apply_multi")) return rc;
+  if (n_targets < 1 || n_targets > MLORA_MAX_TARGETS || !targets)
+    return fail(MLORA_ERR_INVALID, "lora_apply_multi: n_targets=%d outside [1,%d]", n_targets, MLORA_MAX_TARGETS);
+  if (T == 0) return MLORA_OK;
+  if (!x || !scratch || !scales) return fail(MLORA_ERR_INVALID, "lora_apply_multi: null pointer");
+  if (!aligned16(x) || !aligned16(scratch)) return fail(MLORA_ERR_INVALID, "lora_apply_multi: x and scratch must be 16-byte aligned");
+  for (int i = 0; i < n_targets; ++i) {
+    if (!targets[i].y || !targets[i].w_b || !aligned16(targets[i].y) || !aligned16(targets[i].w_b))
+      return fail(MLORA_ERR_INVALID, "lora_apply_multi: target %d has a null or misaligned pointer", i);
+    if (targets[i].slot < 0 || targets[i].slot >= pool_a->n_slots)
+      return fail(MLORA_ERR_INVALID, "lora_apply_multi: target %d slot %d outside [0,%d)", i, targets[i].slot, pool_a->n_slots);
+    for (int j = 0; j < i; ++j)
+      if (targets[j].y == targets[i].y) return fail(MLORA_ERR_INVALID, "lora_apply_multi: targets %d and %d share y", j, i);
+  }
+  if (ksplit == 0) ksplit = default_ksplit(T, plan->n_adapters, plan->bm_shrink, h_in);
+  if (ksplit < 1 || ksplit > 64) return fail(MLORA_ERR_INVALID, "lora_apply_multi: ksplit=%d outside [1,64]", ksplit);
+  const size_t per_target = scratch_bytes(T, max_rank, ksplit);
+  if (scratch_nbytes < per_target * (size_t)n_targets)
+    return fail(MLORA_ERR_WORKSPACE, "lora_apply_multi: scratch has %zu bytes, needs %zu", scratch_nbytes,
+                per_target * (size_t)n_targets);
+  const PlanLayout L = plan_layout(plan->T, plan->n_adapters);
+  const int64_t rp = partial_stride(max_rank);
+  const int64_t v_bytes = align_up(T * rp * 2, 256);
+  const bool rie = ksplit > 1 && (flags & MLORA_REDUCE_IN_EXPAND);
+  ShrinkArgs a;
+  a.plan = static_cast<const int32_t *>(plan->dev);
+  a.off_perm = L.off_perm;
+  a.off_tiles = L.off_tiles_s;
+  a.off_prank = L.off_prank;
+  a.partial = reinterpret_cast<float *>(static_cast<char *>(scratch) + v_bytes);
+  a.x = static_cast<const uint16_t *>(x);
+  a.pool = pool_dev(pool_a);
+  a.T = (int)T;
+  a.h_in = (int)h_in;
+  a.rp = (int)rp;
+  a.slot = targets[0].slot;
+  a.ksplit = ksplit;
+  a.kchunk = (int)align_up((h_in + ksplit - 1) / ksplit, 128);
+  a.out = static_cast<uint16_t *>(scratch);
+  a.out_stride = rp;
+  a.out_by_token = 0;
+  a.mode = MLORA_SHRINK_OVERWRITE;
+  a.width = 0;
+  a.ncols = (int)rp;
+  a.partial_only = rie ? 1 : 0;
+  a.n_targets = n_targets;
+  for (int i = 0; i < MLORA_MAX_TARGETS; ++i) a.slots[i] = targets[i < n_targets ? i : 0].slot;
+  a.out_tstride = (int64_t)(per_target / 2);
+  a.partial_tstride = (int64_t)(per_target / 4);
+  if (int rc = launch_shrink((hipStream_t)stream, a, plan->bm_shrink, (int)max_rank,
+                             tiles_upper(T, plan->n_adapters, plan->bm_shrink), dtype))
+    return rc;
+  if (ksplit > 1 && !rie)
+    if (int rc = launch_shrink_reduce((hipStream_t)stream, a, dtype)) return rc;
+
+  ExpandArgs e;
+  e.plan = a.plan;
+  e.off_perm = L.off_perm;
+  e.off_tiles = L.off_tiles_e;
+  e.y = static_cast<uint16_t *>(targets[0].y);
+  e.v = static_cast<const uint16_t *>(scratch);
+  e.v_stride = rp;
+  e.v_by_pos = 1;
+  e.partial = rie ? a.partial : nullptr;
+  e.ksplit = rie ? ksplit : 1;
+  e.rp = (int)rp;
+  e.pool = pool_dev(pool_a);
+  e.scales = static_cast<const uint16_t *>(scales);
+  e.T = (int)T;
+  e.h_out = (int)h_out;
+  e.kmax = (int)max_rank;
+  e.slot = targets[0].slot;
+  e.n_ochunks = (int)((h_out + expand_bn() - 1) / expand_bn());
+  e.n_targets = n_targets;
+  for (int i = 0; i < MLORA_MAX_TARGETS; ++i) {
+    const mlora_target &t = targets[i < n_targets ? i : 0];
+    e.slots[i] = t.slot;
+    e.ys[i] = static_cast<uint16_t *>(t.y);
+    e.ws[i] = static_cast<const uint16_t *>(t.w_b);
+    e.w_rows_t[i] = t.w_b_rows;
+  }
+  e.v_tstride = a.out_tstride;
+  e.partial_tstride = a.partial_tstride;
+  return launch_expand((hipStream_t)stream, e, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand), dtype);
 }
 
 int mlora_lora_fused(void *stream, const mlora_plan *plan, void *y, const void *x, int64_t T, int64_t h_in,

@@ -26,8 +26,21 @@ constexpr int STAGE_LD = EXP_WN + 4;
 constexpr int EXP_MBU = 2;         // 16-token blocks whose loads are in flight together
 constexpr int EXP_MAX_BM = 256;   // tallest expand tile (tokens), one thread per token at set-up
 
+// the arguments of target z of a multi-target launch
+__device__ __forceinline__ ExpandArgs select_target(const ExpandArgs &a, int z) {
+  ExpandArgs p = a;
+  p.slot = a.slots[z];
+  p.y = a.ys[z];
+  p.pool.w = a.ws[z];
+  p.pool.w_rows = a.w_rows_t[z];
+  p.v = a.v + (int64_t)z * a.v_tstride;
+  if (a.partial) p.partial = a.partial + (int64_t)z * a.partial_tstride;
+  return p;
+}
+
 template <typename T, int KB, bool PARTIAL>
-__global__ __launch_bounds__(256) void expand_kernel(ExpandArgs p) {
+__global__ __launch_bounds__(256) void expand_kernel(ExpandArgs args_in) {
+  const ExpandArgs p = select_target(args_in, blockIdx.y);
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   __shared__ float stage[4][16][STAGE_LD];
@@ -212,7 +225,7 @@ int launch_expand(hipStream_t st, const ExpandArgs &a, int max_rank, int64_t gri
   if (grid_tiles <= 0) return MLORA_OK;
   const int64_t blocks = grid_tiles * a.n_ochunks;
   if (blocks > 0x7fffffff) return fail(MLORA_ERR_NO_KERNEL, "expand: grid too large");
-  dim3 grid((unsigned)blocks);
+  dim3 grid((unsigned)blocks, (unsigned)a.n_targets);
   return dt == MLORA_F16 ? launch_expand_t<_Float16>(st, a, kb, grid)
                          : launch_expand_t<__bf16>(st, a, kb, grid);
 }

@@ -83,6 +83,10 @@ struct ShrinkArgs {
   int T, h_in, rp, slot, ksplit, kchunk;
   int out_by_token, mode, width, ncols;
   int partial_only;           // leave the K-chunk partials for the expand to sum (no reduce launch)
+  // several targets that share x in one launch (grid z = target): slot, v buffer and partials per target
+  int n_targets;
+  int slots[MLORA_MAX_TARGETS];
+  int64_t out_tstride, partial_tstride;   // elements / floats between consecutive targets
 };
 
 struct ExpandArgs {
@@ -94,6 +98,13 @@ struct ExpandArgs {
   int v_by_pos;               // rows indexed by sorted position (internal buffer) or by token
   const float *partial;       // when set: v = T(sum_s partial[s][pos][:]) with ksplit chunks of T*rp floats
   int ksplit, rp;
+  // several targets in one launch (grid y = target)
+  int n_targets;
+  int slots[MLORA_MAX_TARGETS];
+  uint16_t *ys[MLORA_MAX_TARGETS];
+  const uint16_t *ws[MLORA_MAX_TARGETS];
+  int64_t w_rows_t[MLORA_MAX_TARGETS];
+  int64_t v_tstride, partial_tstride;
   PoolDev pool;
   const uint16_t *scales;
   int T, h_out, kmax, slot, n_ochunks;

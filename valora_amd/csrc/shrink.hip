@@ -20,6 +20,15 @@ namespace mlora {
 
 namespace {
 
+// the arguments of target z of a multi-target launch
+__device__ __forceinline__ ShrinkArgs select_target(const ShrinkArgs &a, int z) {
+  ShrinkArgs p = a;
+  p.slot = a.slots[z];
+  p.out = a.out + (int64_t)z * a.out_tstride;
+  p.partial = a.partial + (int64_t)z * a.partial_tstride;
+  return p;
+}
+
 template <typename T>
 __device__ __forceinline__ void store_v(const ShrinkArgs &p, int pos, int t, int r, int col, float v) {
   using Tr = Traits<T>;
@@ -73,7 +82,8 @@ __device__ __forceinline__ void shrink_epilogue(const ShrinkArgs &p, const float
 // v[row, :] = T(sum_s partial[s][row][:]) for every row that has an adapter; one thread per four
 // columns, every chunk requested before any is consumed.
 template <typename T>
-__global__ __launch_bounds__(256) void shrink_reduce_kernel(ShrinkArgs p) {
+__global__ __launch_bounds__(256) void shrink_reduce_kernel(ShrinkArgs args_in) {
+  const ShrinkArgs p = select_target(args_in, blockIdx.y);
   const int n_active = p.plan[H_NACTIVE];
   const int quarter = p.rp >> 2;
   const int64_t total = (int64_t)n_active * quarter;
@@ -99,7 +109,8 @@ __global__ __launch_bounds__(256) void shrink_reduce_kernel(ShrinkArgs p) {
 }
 
 template <typename T, int MB, int NB>
-__global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs p) {
+__global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs args_in) {
+  const ShrinkArgs p = select_target(args_in, blockIdx.z);
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   constexpr int NBLK = MB * NB;
@@ -230,7 +241,8 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs p) {
 // operand read is ds_read_b128 at lane*16 -- conflict free, no layout conversion.  Two stages
 // are always in flight while the third is consumed; one s_barrier per K step.
 template <typename T, int NB>
-__global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs p) {
+__global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
+  const ShrinkArgs p = select_target(args_in, blockIdx.z);
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   constexpr int MBW = 2, KC = 64, KS = KC / 32, STAGES = 3;
@@ -429,9 +441,9 @@ int launch_shrink_reduce(hipStream_t st, const ShrinkArgs &a, mlora_dtype dt) {
   if (blocks > 2048) blocks = 2048;
   if (blocks < 1) blocks = 1;
   if (dt == MLORA_F16)
-    hipLaunchKernelGGL(shrink_reduce_kernel<_Float16>, dim3((unsigned)blocks), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(shrink_reduce_kernel<_Float16>, dim3((unsigned)blocks, (unsigned)a.n_targets), dim3(256), 0, st, a);
   else
-    hipLaunchKernelGGL(shrink_reduce_kernel<__bf16>, dim3((unsigned)blocks), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(shrink_reduce_kernel<__bf16>, dim3((unsigned)blocks, (unsigned)a.n_targets), dim3(256), 0, st, a);
   return check_launch("shrink_reduce_kernel");
 }
 
@@ -441,7 +453,7 @@ int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int
   nb = nb <= 1 ? 1 : nb <= 2 ? 2 : nb <= 4 ? 4 : 8;
   if (nb == 8 && bm == 64) return fail(MLORA_ERR_NO_KERNEL, "shrink: rank > 64 needs tile height 16, 32 or 128");
   if (grid_tiles <= 0) return MLORA_OK;
-  dim3 grid((unsigned)grid_tiles, (unsigned)a.ksplit);
+  dim3 grid((unsigned)grid_tiles, (unsigned)a.ksplit, (unsigned)a.n_targets);
   return dt == MLORA_F16 ? launch_shrink_t<_Float16>(st, a, bm, nb, grid)
                          : launch_shrink_t<__bf16>(st, a, bm, nb, grid);
 }

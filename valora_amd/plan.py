@@ -119,6 +119,34 @@ class LoraPlan:
             None, 0, self.max_rank, pb, int(slot), _lib.ptr(scales), int(self.ksplit), self.flags,
             _lib.dtype_code(y.dtype)))
 
+    def apply_multi(self, ys, x: torch.Tensor, key_buffer: torch.Tensor, value_buffers, a_start: torch.Tensor,
+                    a_len: torch.Tensor, a_loc: torch.Tensor, slots, scales: torch.Tensor) -> None:
+        """Several targets that read the same ``x`` (q, k, v of a layer; gate and up) in two launches:
+        ``ys[i] += scale_a * (x @ A_a[slots[i]].T) @ B_a[slots[i]]``.  ``value_buffers`` is one pool tensor or
+        one per target.  Same results as ``apply`` called once per target."""
+        n = len(ys)
+        if not 1 <= n <= _lib.MAX_TARGETS or len(slots) != n:
+            raise RuntimeError(f"apply_multi takes 1..{_lib.MAX_TARGETS} targets with one slot each")
+        vbs = list(value_buffers) if isinstance(value_buffers, (list, tuple)) else [value_buffers] * n
+        h_in, h_out = x.size(1), ys[0].size(1)
+        for y, vb in zip(ys, vbs):
+            self._check(x, y, key_buffer, vb)
+            if y.size(1) != h_out:
+                raise RuntimeError("all targets of one call must have the same output width")
+        if scales.dtype != x.dtype:
+            scales = scales.to(x.dtype)
+        need = n * int(_lib.lib().mlora_scratch_bytes(self.T, self.max_rank, self.ksplit))
+        if self.scratch.numel() < need:
+            self.scratch = torch.empty(need, dtype=torch.uint8, device=self.device)
+        pa = _lib.make_pool(key_buffer, a_start, a_len, a_loc, h_in, self.n_slots)
+        tg = (_lib.Target * n)()
+        for i in range(n):
+            tg[i] = _lib.Target(_lib.ptr(ys[i]), _lib.ptr(vbs[i]), vbs[i].numel() // h_out, int(slots[i]))
+        _lib.check(_lib.lib().mlora_lora_apply_multi(
+            _lib.current_stream(self.device), self.handle, _lib.ptr(self.scratch), self.scratch.numel(), _lib.ptr(x),
+            self.T, h_in, h_out, self.max_rank, pa, n, tg, _lib.ptr(scales), int(self.ksplit), self.flags,
+            _lib.dtype_code(x.dtype)))
+
     def apply_fused(self, y: torch.Tensor, x: torch.Tensor, key_buffer: torch.Tensor, value_buffer: torch.Tensor,
                     a_start: torch.Tensor, a_len: torch.Tensor, a_loc: torch.Tensor, slot: int,
                     scales: torch.Tensor, replicas: int = 0) -> None:
