@@ -479,6 +479,7 @@ int mlora_lora_fused(void *stream, const mlora_plan *plan, void *y, const void *
   a.h_out = (int)h_out;
   a.kmax = (int)max_rank;
   a.slot = slot;
+  a.tiles = (int)tiles;
   a.tiles_pad = (int)align_up(tiles, 8);  // replicas of a tile land on the same XCD (workgroup id mod 8)
   a.o_per_wg = (int)align_up((h_out + replicas - 1) / replicas, 64);
   return launch_fused((hipStream_t)stream, a, (int)max_rank, replicas, dtype);

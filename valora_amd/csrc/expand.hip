@@ -46,12 +46,11 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs args_in) {
   __shared__ float stage[4][16][STAGE_LD];
   __shared__ int32_t s_perm[EXP_MAX_BM];
 
-  const int32_t *__restrict__ hdr = p.plan;
   const int tile_idx = blockIdx.x / p.n_ochunks;
   const int oc = blockIdx.x - tile_idx * p.n_ochunks;
-  if (tile_idx >= hdr[H_NTILES_E]) return;
   const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int a = tile[0], r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
+  if (cnt <= 0) return;   // records past the last tile are zero
   const int rk = min(r, p.kmax);  // rank columns the narrow operand really has (bgmv_impl.cuh:167,186)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;

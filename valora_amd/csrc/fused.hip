@@ -39,12 +39,12 @@ __global__ __launch_bounds__(FT) void fused_kernel(FusedArgs p) {
   __shared__ uint16_t s_v[16][RP + 8];
   __shared__ int32_t s_perm[16];
 
-  const int32_t *__restrict__ hdr = p.plan;
   const int tile_idx = blockIdx.x % p.tiles_pad;
   const int rep = blockIdx.x / p.tiles_pad;
-  if (tile_idx >= hdr[H_NTILES_S]) return;
+  if (tile_idx >= p.tiles) return;
   const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int a = tile[0], r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
+  if (cnt <= 0) return;   // records past the last tile are zero
   const int rk = min(r, p.kmax);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;

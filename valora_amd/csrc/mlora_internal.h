@@ -117,7 +117,7 @@ struct FusedArgs {
   const uint16_t *x;
   PoolDev pa, pb;
   const uint16_t *scales;
-  int T, h_in, h_out, kmax, slot, tiles_pad, o_per_wg;
+  int T, h_in, h_out, kmax, slot, tiles, tiles_pad, o_per_wg;   // tiles: records in the list; tiles_pad: rounded up to 8
 };
 
 int launch_fused(hipStream_t st, const FusedArgs &a, int max_rank, int replicas, mlora_dtype dt);

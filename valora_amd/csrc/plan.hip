@@ -183,6 +183,14 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
       tl[4] = (int32_t)st;
       tl[5] = 0; tl[6] = 0; tl[7] = 0;
     }
+    // the kernels' grids are sized with the upper bound of the tile count: records past the last
+    // tile say "no tokens", so a workgroup needs no second look-up to know that it has nothing to do
+    const int upper = (T + bm - 1) / bm + min(A, T);
+    for (int i = n_tiles + tid; i < upper; i += PLAN_THREADS) {
+      int32_t *tl = tiles + (int64_t)i * TILE_WORDS;
+#pragma unroll
+      for (int k = 0; k < TILE_WORDS; ++k) tl[k] = 0;
+    }
   }
   __syncthreads();
   if (tid == 0) {
