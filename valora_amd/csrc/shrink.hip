@@ -125,11 +125,13 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs args_in) {
   constexpr int NBLK = MB * NB;
   __shared__ float red[2][NBLK * 256];
 
-  const int tile_idx = blockIdx.x;
+  // the K chunk is the fast index: workgroup id mod 8 selects the XCD, so the tiles of an adapter
+  // that share a K chunk of A meet in one L2
+  const int tile_idx = blockIdx.x / p.ksplit;
   const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
-  const int s = blockIdx.y;
+  const int s = blockIdx.x - tile_idx * p.ksplit;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lrow = lane & 15, kg = lane >> 4;
@@ -244,9 +246,11 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs args_in) {
 // operands of a 64-wide K step go from global memory straight into LDS with 16-byte
 // global_load_lds (no registers are held while the data is in flight): every wave streams its
 // own x rows into a private part of the stage, the adapter's A rows are loaded once per
-// workgroup and shared by all waves.  A load instruction writes 1 KB to LDS in lane order, and
-// each lane asks for exactly the 16 bytes it will later feed to the matrix core, so the MFMA
-// operand read is ds_read_b128 at lane*16 -- conflict free, no layout conversion.  Two stages
+// workgroup and shared by all waves.  A load instruction covers 8 rows x 128 contiguous bytes
+// (whole cache lines: asking for the two halves of a line with two instructions measured up to
+// 30 % slower) and writes them to LDS in lane order, so a stage holds rows of 128 bytes; the
+// lane that fills 16-byte chunk c of row R fetches global chunk c ^ (R & 7), which spreads the
+// later ds_read_b128 of an MFMA operand (16 rows, one chunk column) over the banks.  Two stages
 // are always in flight while the third is consumed; one s_barrier per K step.
 template <typename T, int NB>
 __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
@@ -254,9 +258,10 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   constexpr int MBW = 2, KC = 64, KS = KC / 32, STAGES = 3;
-  constexpr int XBLK = MBW * KS;                        // 1 KB blocks of x per wave per stage
-  constexpr int ABLK = NB * KS;                         // 1 KB blocks of A per stage (shared)
-  constexpr int APW = ABLK >= 4 ? ABLK / 4 : 1;         // A blocks each wave loads per stage
+  static_assert(KC * 2 == 128, "a K step is one 128-byte line per row");
+  constexpr int XBLK = MBW * 2;                         // 8-row groups (1 KB) of x per wave per stage
+  constexpr int ABLK = NB * 2;                          // 8-row groups of A per stage (shared)
+  constexpr int APW = ABLK >= 4 ? ABLK / 4 : 1;         // A groups each wave loads per stage
   constexpr int A_SLOTS = APW * 4;                      // >= ABLK; surplus slots hold duplicates
   constexpr int STAGE_BYTES = (4 * XBLK + A_SLOTS) * 1024;
   constexpr int TILE_BYTES = 128 * NB * 16 * 4;
@@ -264,54 +269,57 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
   constexpr int RING_BYTES = STAGES * STAGE_BYTES + 1024;   // + one scratch block for dummy loads
   __shared__ __align__(16) unsigned char s_raw[RING_BYTES > TILE_BYTES ? RING_BYTES : TILE_BYTES];
 
-  const int tile_idx = blockIdx.x;
+  // the K chunk is the fast index: workgroup id mod 8 selects the XCD, so the tiles of an adapter
+  // that share a K chunk of A meet in one L2
+  const int tile_idx = blockIdx.x / p.ksplit;
   TRACE_T(0);
   const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
-  const int s = blockIdx.y;
+  const int s = blockIdx.x - tile_idx * p.ksplit;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int lrow = lane & 15, kg = lane >> 4;
+  const int lrow = lane & 15, kg = lane >> 4;           // MFMA operand roles
+  const int grow = lane >> 3;                           // loader roles: row within an 8-row group,
+  const int gchunk = (lane & 7) ^ grow;                 // global 16-byte chunk this lane fetches
   const int32_t *__restrict__ perm = p.plan + p.off_perm;
   const int64_t base = (int64_t)astart + (int64_t)r * p.slot;
   const int wrow0 = wave * 16 * MBW;
   const bool wave_active = wrow0 < cnt;                 // wave-uniform
 
-  // this lane's global row pointers
-  const uint16_t *xp[MBW];
-  bool xok[MBW];
+  // this lane's global row pointers (already at its chunk)
+  const uint16_t *xp[XBLK];
+  bool xok[XBLK];
 #pragma unroll
-  for (int mb = 0; mb < MBW; ++mb) {
-    const int row = wrow0 + mb * 16 + lrow;
-    xok[mb] = row < cnt;
-    const int t = xok[mb] ? perm[pos0 + row] : 0;
-    xp[mb] = p.x + (int64_t)t * p.h_in;
+  for (int g = 0; g < XBLK; ++g) {
+    const int row = wrow0 + g * 8 + grow;
+    xok[g] = row < cnt;
+    const int t = xok[g] ? perm[pos0 + row] : 0;
+    xp[g] = p.x + (int64_t)t * p.h_in + gchunk * 8;
   }
-  // A blocks this wave loads: slot = wave*APW + i -> (nb, ks) = (slot / KS, slot % KS) when slot < ABLK
+  // A groups this wave loads: slot = wave*APW + i -> rows slot*8 .. slot*8+7 of the rank
   const uint16_t *ap[APW];
   bool aok[APW];
-  int aks[APW];
 #pragma unroll
   for (int i = 0; i < APW; ++i) {
-    const int slot = (wave * APW + i) % ABLK;           // surplus slots duplicate real blocks
-    const int nb = slot / KS;
-    aks[i] = slot % KS;
-    const int j = nb * 16 + lrow;
+    const int slot = (wave * APW + i) % ABLK;           // surplus slots duplicate real groups
+    const int j = slot * 8 + grow;
     const int64_t idx = base + j;
     bool ok = j < r && idx >= 0 && idx < p.pool.a_loc_len;
     const int64_t prow = ok ? p.pool.a_loc[idx] : 0;
     ok = ok && prow >= 0 && prow < p.pool.w_rows;
     aok[i] = ok;
-    ap[i] = p.pool.w + (ok ? prow : 0) * p.h_in;
+    ap[i] = p.pool.w + (ok ? prow : 0) * p.h_in + gchunk * 8;
   }
 
   const int kbeg = s * p.kchunk;
   const int kend = min(p.h_in, kbeg + p.kchunk);
   const int n_steps = (kend - kbeg + KC - 1) / KC;
 
-  auto lds_x = [&](int stage, int blk) { return s_raw + stage * STAGE_BYTES + (wave * XBLK + blk) * 1024; };
-  auto lds_a = [&](int stage, int slot) { return s_raw + stage * STAGE_BYTES + (4 * XBLK + slot) * 1024; };
+  // byte offsets inside a stage: x rows of this wave, then the shared A rows
+  const uint32_t ring = lds_offset(s_raw);
+  const uint32_t x_off = (uint32_t)(wave * XBLK) * 1024u;
+  const uint32_t a_off = (uint32_t)(4 * XBLK) * 1024u;
   const u32x4 zero4 = {0, 0, 0, 0};
 
   // Issue every load of one K step: EXACTLY LOADS_PER_STAGE load instructions per wave, because the
@@ -328,23 +336,29 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
   };
   auto issue = [&](int step) {
     const int stage = step % STAGES;
-    const int k0 = kbeg + step * KC;
+    const int k = kbeg + step * KC + gchunk * 8;        // first K element of this lane's chunk
+    const bool kok = k < kend;
+    unsigned char *sbase = s_raw + stage * STAGE_BYTES;
 #pragma unroll
-    for (int mb = 0; mb < MBW; ++mb)
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int k = k0 + ks * 32 + kg * 8;
-        unsigned char *dst = lds_x(stage, mb * KS + ks);
-        load_or_dummy(xok[mb] && k < kend, xp[mb] + k, dst);
-        if (k >= kend) lds_write16(lds_offset(dst) + lane * 16, zero4);
-      }
+    for (int g = 0; g < XBLK; ++g) {
+      unsigned char *dst = sbase + x_off + g * 1024;
+      load_or_dummy(xok[g] && kok, xp[g] + kbeg + step * KC, dst);
+      if (!kok) lds_write16(lds_offset(dst) + lane * 16, zero4);
+    }
 #pragma unroll
     for (int i = 0; i < APW; ++i) {
-      const int k = k0 + aks[i] * 32 + kg * 8;
-      unsigned char *dst = lds_a(stage, wave * APW + i);
-      load_or_dummy(aok[i] && k < kend, ap[i] + k, dst);
-      if (k >= kend) lds_write16(lds_offset(dst) + lane * 16, zero4);
+      unsigned char *dst = sbase + a_off + (wave * APW + i) * 1024;
+#ifdef MLORA_EXP_NOA
+      load_or_dummy(false, ap[i] + kbeg + step * KC, dst);
+#else
+      load_or_dummy(aok[i] && kok, ap[i] + kbeg + step * KC, dst);
+#endif
+      if (!kok) lds_write16(lds_offset(dst) + lane * 16, zero4);
     }
+  };
+  // where the MFMA operand (row R of a region, K block ks) of this lane sits inside a stage
+  auto frag_off = [&](int R, int ks) -> uint32_t {
+    return (uint32_t)R * 128u + (uint32_t)(((ks * 4 + kg) ^ (R & 7)) * 16);
   };
 
   f32x4 acc[MBW][NB];
@@ -362,18 +376,26 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
     // iteration is free to be refilled
     if (step + 1 < n_steps) wait_vmcnt<LOADS_PER_STAGE>(); else wait_vmcnt<0>();
     wait_lgkmcnt0();
+#ifndef MLORA_EXP_NOBARRIER
     __builtin_amdgcn_s_barrier();
+#endif
     if (step == 0) TRACE_T(4);
     if (step + 2 < n_steps) issue(step + 2);
     const int stage = step % STAGES;
+#ifdef MLORA_EXP_NOCOMPUTE
+    if (false) {
+#else
     if (wave_active) {
+#endif
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         u32x4 xf[MBW], bf[NB];
 #pragma unroll
-        for (int mb = 0; mb < MBW; ++mb) xf[mb] = lds_read16(lds_offset(lds_x(stage, mb * KS + ks)) + lane * 16);
+        for (int mb = 0; mb < MBW; ++mb)
+          xf[mb] = lds_read16(ring + stage * STAGE_BYTES + x_off + frag_off(mb * 16 + lrow, ks));
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) bf[nb] = lds_read16(lds_offset(lds_a(stage, nb * KS + ks)) + lane * 16);
+        for (int nb = 0; nb < NB; ++nb)
+          bf[nb] = lds_read16(ring + stage * STAGE_BYTES + a_off + frag_off(nb * 16 + lrow, ks));
         wait_lgkmcnt0();
 #pragma unroll
         for (int mb = 0; mb < MBW; ++mb) pin(xf[mb]);
@@ -474,7 +496,8 @@ int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int
   nb = nb <= 1 ? 1 : nb <= 2 ? 2 : nb <= 4 ? 4 : 8;
   if (nb == 8 && bm == 64) return fail(MLORA_ERR_NO_KERNEL, "shrink: rank > 64 needs tile height 16, 32 or 128");
   if (grid_tiles <= 0) return MLORA_OK;
-  dim3 grid((unsigned)grid_tiles, (unsigned)a.ksplit, (unsigned)a.n_targets);
+  if (grid_tiles * a.ksplit > 0x7fffffff) return fail(MLORA_ERR_NO_KERNEL, "shrink: grid too large");
+  dim3 grid((unsigned)(grid_tiles * a.ksplit), 1, (unsigned)a.n_targets);
   return dt == MLORA_F16 ? launch_shrink_t<_Float16>(st, a, bm, nb, grid)
                          : launch_shrink_t<__bf16>(st, a, bm, nb, grid);
 }
