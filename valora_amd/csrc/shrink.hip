@@ -119,19 +119,21 @@ __global__ __launch_bounds__(256) void shrink_reduce_kernel(ShrinkArgs args_in) 
 
 template <typename T, int MB, int NB>
 __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs args_in) {
-  const ShrinkArgs p = select_target(args_in, blockIdx.z);
+  // workgroup id = (tile * targets + target) * ksplit + K chunk.  The id mod 8 selects the XCD, so
+  // with the K chunk as the fast index the tiles of an adapter that share a K chunk of A, and the
+  // targets that share a K chunk of x, meet in one L2.
+  const int wg_tz = blockIdx.x / args_in.ksplit;
+  const int tile_idx = wg_tz / args_in.n_targets;
+  const ShrinkArgs p = select_target(args_in, wg_tz - tile_idx * args_in.n_targets);
+  const int s = blockIdx.x - wg_tz * p.ksplit;
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   constexpr int NBLK = MB * NB;
   __shared__ float red[2][NBLK * 256];
 
-  // the K chunk is the fast index: workgroup id mod 8 selects the XCD, so the tiles of an adapter
-  // that share a K chunk of A meet in one L2
-  const int tile_idx = blockIdx.x / p.ksplit;
   const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
-  const int s = blockIdx.x - tile_idx * p.ksplit;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lrow = lane & 15, kg = lane >> 4;
@@ -254,7 +256,13 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs args_in) {
 // are always in flight while the third is consumed; one s_barrier per K step.
 template <typename T, int NB>
 __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
-  const ShrinkArgs p = select_target(args_in, blockIdx.z);
+  // workgroup id = (tile * targets + target) * ksplit + K chunk.  The id mod 8 selects the XCD, so
+  // with the K chunk as the fast index the tiles of an adapter that share a K chunk of A, and the
+  // targets that share a K chunk of x, meet in one L2.
+  const int wg_tz = blockIdx.x / args_in.ksplit;
+  const int tile_idx = wg_tz / args_in.n_targets;
+  const ShrinkArgs p = select_target(args_in, wg_tz - tile_idx * args_in.n_targets);
+  const int s = blockIdx.x - wg_tz * p.ksplit;
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   constexpr int MBW = 2, KC = 64, KS = KC / 32, STAGES = 3;
@@ -269,14 +277,10 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
   constexpr int RING_BYTES = STAGES * STAGE_BYTES + 1024;   // + one scratch block for dummy loads
   __shared__ __align__(16) unsigned char s_raw[RING_BYTES > TILE_BYTES ? RING_BYTES : TILE_BYTES];
 
-  // the K chunk is the fast index: workgroup id mod 8 selects the XCD, so the tiles of an adapter
-  // that share a K chunk of A meet in one L2
-  const int tile_idx = blockIdx.x / p.ksplit;
   TRACE_T(0);
   const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
-  const int s = blockIdx.x - tile_idx * p.ksplit;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lrow = lane & 15, kg = lane >> 4;           // MFMA operand roles
@@ -496,8 +500,8 @@ int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int
   nb = nb <= 1 ? 1 : nb <= 2 ? 2 : nb <= 4 ? 4 : 8;
   if (nb == 8 && bm == 64) return fail(MLORA_ERR_NO_KERNEL, "shrink: rank > 64 needs tile height 16, 32 or 128");
   if (grid_tiles <= 0) return MLORA_OK;
-  if (grid_tiles * a.ksplit > 0x7fffffff) return fail(MLORA_ERR_NO_KERNEL, "shrink: grid too large");
-  dim3 grid((unsigned)(grid_tiles * a.ksplit), 1, (unsigned)a.n_targets);
+  if (grid_tiles * a.ksplit * a.n_targets > 0x7fffffff) return fail(MLORA_ERR_NO_KERNEL, "shrink: grid too large");
+  dim3 grid((unsigned)(grid_tiles * a.ksplit * a.n_targets));
   return dt == MLORA_F16 ? launch_shrink_t<_Float16>(st, a, bm, nb, grid)
                          : launch_shrink_t<__bf16>(st, a, bm, nb, grid);
 }
