@@ -209,8 +209,60 @@ def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph):
                                 "us_per_layer_multi_target": round(fused_total, 2)}
         del wd
         torch.cuda.empty_cache()
+    report["adapter_residency"] = bench_adapter_residency(torch, dev)
     with open(path, "w") as f:
         json.dump(report, f, indent=1)
+
+
+def bench_adapter_residency(torch, dev):
+    """Loading an adapter into the paged pool and dropping adapters again: one rank-64 adapter of a
+    32-layer, 4096-wide model is 2 x 32 x 256 rows of 8 KB (134 MB), moved by one row-scatter launch
+    per buffer; the HBM figure counts every byte read once and written once."""
+    from valora_amd import _lib
+    from valora_amd.infer_adapter import InferAdapter, LoraAdapterWeights, MemoryAllocator
+    net = dict(num_hidden_layers=32, hidden_size=4096, num_attention_heads=32)
+    rows_total = 16384
+    mm = MemoryAllocator(rows_total, 0, torch.float16, 32, 128, 32, dev)
+    out = {}
+    for r in (16, 64):
+        n = 4 * r
+        packed = torch.randn(32, 2, n, 4096, device=dev).to(torch.float16)
+        loc = torch.randperm(rows_total, device=dev)[:n].contiguous()
+        L, st_of = _lib.lib(), _lib.current_stream
+        esz = 2
+
+        def scatter_both():
+            for which, buf in ((0, mm.key_buffer), (1, mm.value_buffer)):
+                _lib.check(L.mlora_pool_scatter_rows(st_of(dev), _lib.ptr(buf), rows_total, rows_total * 4096 * esz,
+                                                     _lib.c_void_p(packed.data_ptr() + which * n * 4096 * esz),
+                                                     2 * n * 4096 * esz, _lib.ptr(loc), n, 4096 * esz, 32))
+
+        ms, _ = time_graph(torch, scatter_both, 20, 3, False)
+        moved = 2 * packed.numel() * esz
+        out[f"load_rank{r}"] = {"us": round(ms * 1e3, 1), "bytes_read_plus_written": moved,
+                                "gbps": round(moved / ms / 1e6, 1), "hbm_frac": round(moved / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                                "launches": 2, "reference_launches": 64}
+    # allocator and re-index latency with 200 resident adapters
+    ia = InferAdapter.init(mm)
+    small = dict(num_hidden_layers=32, hidden_size=4096, num_attention_heads=32)
+    ads = [LoraAdapterWeights(f"a{i}", 16, 32.0, small, torch.zeros(32, 2, 64, 4096, dtype=torch.float16))
+           for i in range(200)]
+    t0 = time.perf_counter()
+    ia.load_adapters(ads)
+    torch.cuda.synchronize()
+    out["load_200_adapters_rank16_ms_wall"] = round((time.perf_counter() - t0) * 1e3, 2)
+    t0 = time.perf_counter()
+    ia.offload_adapters([f"a{i}" for i in range(0, 200, 2)])
+    torch.cuda.synchronize()
+    out["offload_100_of_200_ms_wall"] = round((time.perf_counter() - t0) * 1e3, 3)
+
+    def alloc_free():
+        idx = mm.alloc(256)
+        mm.free(idx)
+
+    ms, _ = time_graph(torch, alloc_free, 50, 3, False)
+    out["alloc256_plus_free_us"] = round(ms * 1e3, 2)
+    return out
 
 
 def main():

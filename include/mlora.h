@@ -210,6 +210,64 @@ int mlora_prefill_expand(void *stream, void *o, const void *x, const mlora_pool 
                          int64_t feat_out, int64_t qkvo, int64_t max_rank, int64_t max_input_len,
                          mlora_dtype dtype, void *workspace, size_t workspace_bytes);
 
+/* ---------------------------------------------------------------------------------------------
+ * Adapter residency: the row allocator of the paged pool, loading / reading back an adapter's rows
+ * and re-indexing when adapters are dropped.  All tensors are device memory; every call only
+ * launches kernels on `stream` (no allocation, no synchronisation).  Integer results are
+ * bit-exact with the reference's tensor code.
+ *
+ * mem_state: one byte per pool row, 1 = free, 0 = taken (the storage of the reference's torch.bool
+ * tensor, valora/common/mem_allocator.py:247).  status: device int32[2] written by the call.
+ * ------------------------------------------------------------------------------------------- */
+
+/* MemoryAllocator.alloc (valora/common/mem_allocator.py:30-56): hands out the first `need` free rows
+ * in index order, writes them ascending to out_index[need] and marks them taken.  The caller keeps
+ * the count of free rows on the host, as the reference does (can_use_mem_size), and only asks for
+ * what is free; status[0] = rows granted (== need then), status[1] = free rows seen by the scan. */
+int mlora_pool_alloc(void *stream, void *mem_state, int64_t tot_size, int64_t need, int64_t *out_index,
+                     int32_t *status);
+
+/* MemoryAllocator.alloc_contiguous (mem_allocator.py:59-75): the first run of `need` consecutive
+ * free rows.  status[0] = first row of the run, or -1 if there is none (state untouched; the
+ * reference returns None). */
+int mlora_pool_alloc_contiguous(void *stream, void *mem_state, int64_t tot_size, int64_t need,
+                                int64_t *out_index, int32_t *status);
+
+/* MemoryAllocator.free (mem_allocator.py:203-217): mem_state[index[i]] = 1. */
+int mlora_pool_free(void *stream, void *mem_state, int64_t tot_size, const int64_t *index, int64_t n);
+
+/* MemoryAllocator.free_all / reset (mem_allocator.py:219-221,246): every row free (or taken). */
+int mlora_pool_fill(void *stream, void *mem_state, int64_t tot_size, int32_t is_free);
+
+/* InferAdapter.load_lora_A / load_lora_B (valora/server/router/model_infer/infer_adapter.py:45-91):
+ * `buffer[layer][loc[i]] = w[layer][i]` for every layer in ONE launch (the reference issues one
+ * indexed assignment per layer and buffer).  pool: [n_layers][pool_rows][row_bytes] with
+ * pool_layer_stride_bytes between layers; packed: [n_layers][n][row_bytes].  Rows and strides are
+ * multiples of 16 bytes.  loc entries outside [0, pool_rows) are skipped. */
+int mlora_pool_scatter_rows(void *stream, void *pool, int64_t pool_rows, int64_t pool_layer_stride_bytes,
+                            const void *packed, int64_t packed_layer_stride_bytes, const int64_t *loc,
+                            int64_t n, int64_t row_bytes, int32_t n_layers);
+
+/* The inverse: `w[layer][i] = buffer[layer][loc[i]]`, the read-back the reference does row-group by
+ * row-group when it densifies an adapter (valora/models/peft/lora_single_batch_infer.py:81-98).
+ * Rows whose loc is outside the pool read as zeros. */
+int mlora_pool_gather_rows(void *stream, const void *pool, int64_t pool_rows, int64_t pool_layer_stride_bytes,
+                           void *packed, int64_t packed_layer_stride_bytes, const int64_t *loc, int64_t n,
+                           int64_t row_bytes, int32_t n_layers);
+
+/* InferAdapter.offload_adapters' re-indexing (infer_adapter.py:218-251 and the var_len_copy kernel
+ * :263-284).  keep[n_keep] = indices of the surviving adapters in the old tensors, ascending.
+ * new_len = old_len[keep]; new_start = exclusive running sum of new_len; new_scaling =
+ * old_scaling[keep] (16-bit elements); new_loc = the surviving a_loc segments, concatenated.  When
+ * mem_state is not null the pool rows of every dropped adapter are freed as well
+ * (infer_adapter.py:214-223).  status[0] = 1 if keep[] held an index outside [0, n_old);
+ * status[1] = entries written to new_loc. */
+int mlora_index_compact(void *stream, const int32_t *keep, int32_t n_keep, int32_t n_old,
+                        const int64_t *old_start, const int64_t *old_len, const int64_t *old_loc,
+                        int64_t old_loc_len, const void *old_scaling, int64_t *new_start, int64_t *new_len,
+                        int64_t *new_loc, int64_t new_loc_len, void *new_scaling, void *mem_state,
+                        int64_t tot_size, int32_t *status);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,6 +26,8 @@ SYMBOLS = [
     "mlora_ids_from_segments", "mlora_ids_from_requests", "mlora_shrink", "mlora_expand", "mlora_lora_apply",
     "mlora_lora_apply_multi", "mlora_lora_fused", "mlora_dispatch_bgmv",
     "mlora_dispatch_sgmm", "mlora_prefill_shrink", "mlora_prefill_expand",
+    "mlora_pool_alloc", "mlora_pool_alloc_contiguous", "mlora_pool_free", "mlora_pool_fill",
+    "mlora_pool_scatter_rows", "mlora_pool_gather_rows", "mlora_index_compact",
 ]
 
 
@@ -97,6 +99,16 @@ def lib():
     L.mlora_prefill_expand.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_void_p,
                                        c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
                                        c_int64, c_int64, c_int, c_void_p, c_size_t]
+    L.mlora_pool_alloc.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]
+    L.mlora_pool_alloc_contiguous.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]
+    L.mlora_pool_free.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_int64]
+    L.mlora_pool_fill.argtypes = [c_void_p, c_void_p, c_int64, c_int32]
+    for n in ("mlora_pool_scatter_rows", "mlora_pool_gather_rows"):
+        getattr(L, n).argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int64,
+                                  c_int64, c_int32]
+    L.mlora_index_compact.argtypes = [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
+                                      c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
+                                      c_void_p]
     for n in SYMBOLS[5:]:  # everything after the size queries returns a status
         getattr(L, n).restype = c_int
     _lib = L
