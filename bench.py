@@ -47,6 +47,8 @@ def parse():
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="first run one plain device copy of this many MiB: a kernel of known traffic to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings with")
+    ap.add_argument("--only-config", type=int, default=0,
+                    help="with --all-configs: report this benchmark configuration only (1, 3, 4 or 5)")
     ap.add_argument("--all-configs", metavar="FILE", default=None,
                     help="also measure every target of configs 1,3,4,5 and write a JSON report to FILE")
     return ap.parse_args()
@@ -140,12 +142,12 @@ def cpu_baseline(torch, w, budget_s=15.0):
                       f"median; {kind}; min {times[0] * 1e6:.1f} us"}
 
 
-def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph):
+def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0):
     """Per-target timing of the other benchmark configurations (report only; the JSON line of the
     default run is config 2).  Each target's shrink+expand is replayed back to back on `reps`
     copies of y so that the read-modify-write does not hit the same lines."""
     report = {}
-    for n in (1, 3, 4, 5):
+    for n in ((only,) if only else (1, 3, 4, 5)):
         w = W.CONFIGS[n]()
         wd = w.to(dev)
         R = max(w.targets[0].pool.ranks)
@@ -209,7 +211,8 @@ def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph):
                                 "us_per_layer_multi_target": round(fused_total, 2)}
         del wd
         torch.cuda.empty_cache()
-    report["adapter_residency"] = bench_adapter_residency(torch, dev)
+    if not only:
+        report["adapter_residency"] = bench_adapter_residency(torch, dev)
     with open(path, "w") as f:
         json.dump(report, f, indent=1)
 
@@ -382,7 +385,7 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, w)
     if args.all_configs:
-        bench_all_configs(torch, W, LoraPlan, dev, args.all_configs, use_graph)
+        bench_all_configs(torch, W, LoraPlan, dev, args.all_configs, use_graph, args.only_config)
     print(json.dumps(out))
 
 
