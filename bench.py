@@ -265,6 +265,28 @@ def bench_adapter_residency(torch, dev):
 
     ms, _ = time_graph(torch, alloc_free, 50, 3, False)
     out["alloc256_plus_free_us"] = round(ms * 1e3, 2)
+
+    # merging one adapter into the q, k, v, o weights of a layer (4 x [4096, 4096]): every weight element
+    # is read once and written once
+    from valora_amd.merge import merge_adapter
+    ia2 = InferAdapter.init(mm)
+    for r in (16, 64):
+        ad = LoraAdapterWeights.dummy(f"m{r}", r, 2.0 * r, net, pin=False)
+        ia2.load_adapters([ad])
+        idx = ia2.idx_map[f"m{r}"]
+        wsets = [[torch.randn(4096, 4096, device=dev).to(torch.float16) for _ in range(4)] for _ in range(3)]
+        state = {"i": 0}
+
+        def merge_layer():
+            ws = wsets[state["i"] % 3]
+            state["i"] += 1
+            merge_adapter(ws, mm.key_buffer[0], mm.value_buffer[0], ia2.a_start, ia2.a_len, ia2.a_loc, idx, 2.0, r)
+
+        ms, _ = time_graph(torch, merge_layer, 30, 3, False)
+        moved = 4 * 2 * 4096 * 4096 * 2
+        out[f"merge_layer_rank{r}"] = {"us": round(ms * 1e3, 1), "bytes_read_plus_written": moved,
+                                       "gbps": round(moved / ms / 1e6, 1),
+                                       "hbm_frac": round(moved / ms / 1e6 / HBM_PEAK_GBPS, 4), "launches": 1}
     return out
 
 

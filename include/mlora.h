@@ -268,6 +268,23 @@ int mlora_index_compact(void *stream, const int32_t *keep, int32_t n_keep, int32
                         int64_t *new_loc, int64_t new_loc_len, void *new_scaling, void *mem_state,
                         int64_t tot_size, int32_t *status);
 
+/* ---------------------------------------------------------------------------------------------
+ * Merging one adapter into the base weights of a layer and taking it out again
+ * (valora/models/peft/lora_single_batch_infer.py:103-149, merge_adapter / unmerge_adapter):
+ *
+ *     w[k][i, o] = T( w[k][i, o] + sign * T( sum_j A[i, j] * T(B[j, o] * scaling) ) ),  k < n_targets
+ *
+ * with A / B the blocks of slot slots[k] of `adapter`, read in place from the key / value pool of
+ * the layer (the reference first copies them into dense matrices, :81-98, and runs a batched GEMM
+ * into a temporary).  w[k] is the [h_in, h_out] row-major weight the base model multiplies with
+ * (x @ W), `ld` elements between rows.  The three rounding points of the reference (scaled B, the
+ * GEMM result, the in-place add) are kept; the accumulation is fp32.  sign = +1 merges, -1
+ * unmerges.  max_rank bounds the adapter's rank (multiple of 8, <= 128).  One launch for all
+ * targets; each weight element is read once and written once. */
+int mlora_merge_adapter(void *stream, void *const *w, const int32_t *slots, int32_t n_targets, int64_t ld,
+                        int64_t h_in, int64_t h_out, const mlora_pool *pool_a, const mlora_pool *pool_b,
+                        int64_t adapter, int64_t max_rank, float scaling, int32_t sign, mlora_dtype dtype);
+
 #ifdef __cplusplus
 }
 #endif

@@ -27,6 +27,12 @@ Pinning status of each function (what fixes it besides its own text):
   the textbook grouped-GEMM closed form it reduces to.
 * ``triton_shrink`` / ``triton_expand`` -- same closed form as ``bgmv_*`` per request;
   pinned by equivalence with ``bgmv_*`` through ``repeat_interleave``.
+* ``merge_weight`` / ``merge_adapter`` -- a library GEMM plus an in-place add in the reference; pinned by
+  small-integer cases where every product and sum is exact (bit-exact against plain Python loops
+  over the pool indices), by fp64, by ``unmerge(merge(W))`` staying within one rounding of W, and by
+  the identity ``x @ merged W == x @ W + lora_op(x)`` to rounding.
+* ``delora_compensate`` -- two applications of ``lora_op``; pinned by the identity
+  ``x @ W_merged + compensate == x @ W + lora_op`` for every token.
 """
 from __future__ import annotations
 
@@ -428,3 +434,47 @@ def rel_l2(a, b) -> float:
     a64, b64 = _f(a, torch.float64), _f(b, torch.float64)
     den = float(b64.norm())
     return float((a64 - b64).norm()) / den if den > 0 else float((a64 - b64).norm())
+
+
+def merge_weight(W: torch.Tensor, A: torch.Tensor, B: torch.Tensor, scaling: float, sign: int = 1) -> torch.Tensor:
+    """``W +- bmm(A, B * scaling)`` with the reference's rounding points: ``b = B * scaling`` is a T
+    tensor, the GEMM accumulates in fp32 and stores T, ``add_`` / ``sub_`` round once more.
+    ``W [H_in, H_out]``, ``A [H_in, r]``, ``B [r, H_out]``.
+
+    valora/models/peft/lora_single_batch_infer.py:113-123 (merge), :137-146 (unmerge).
+    """
+    T = W.dtype
+    b = (B.to(torch.float32) * float(scaling)).to(T)
+    ab = (A.to(torch.float32) @ b.to(torch.float32)).to(T)
+    return (W.to(torch.float32) + float(sign) * ab.to(torch.float32)).to(T)
+
+
+def merge_adapter(weights, kb, vb, a_start, a_len, a_loc, adapter, scaling, slots=(0, 1, 2, 3), n_slots=N_SLOTS,
+                  sign: int = 1):
+    """The four (or fewer) weights of one layer with adapter ``adapter`` merged in (or taken out): A and
+    B of each slot are read back from the pool as the reference does
+    (lora_single_batch_infer.py:81-98: ``key_buffer[loc[s*r:(s+1)*r]].reshape(r, H).T`` and
+    ``value_buffer[...].reshape(H, r).T``).  Returns new tensors."""
+    r = int(a_len[adapter]) // n_slots
+    start = int(a_start[adapter])
+    out = []
+    for W, slot in zip(weights, slots):
+        rows = a_loc[start + slot * r: start + (slot + 1) * r]
+        h_in, h_out = W.shape
+        A = kb.reshape(-1, h_in)[rows].reshape(r, h_in).transpose(0, 1)
+        B = vb.reshape(-1, h_out)[rows].reshape(h_out, r).transpose(0, 1)
+        out.append(merge_weight(W, A, B, scaling, sign))
+    return out
+
+
+def delora_compensate(y, x, kb, vb, a_start, a_len, a_loc, ids, merged, slot, scales, n_slots=N_SLOTS):
+    """While adapter ``merged`` sits in the base weights, tokens of the other adapters get
+    ``+ LoRA(own) - LoRA(merged)``; tokens of the merged adapter and tokens without adapter are
+    left alone.  valora/models/peft/lora_unordered_batch_infer.py:991-1063 (the reference runs the
+    two halves as one doubled batch and adds ``first half - second half``)."""
+    ids = torch.as_tensor(ids, dtype=torch.long)
+    other = (ids != merged) & (ids >= 0) & (ids < a_start.numel())
+    own_ids = torch.where(other, ids, torch.full_like(ids, -1))
+    mrg_ids = torch.where(other, torch.full_like(ids, merged), torch.full_like(ids, -1))
+    y1 = lora_op(y, x, kb, vb, a_start, a_len, a_loc, own_ids, slot, scales, n_slots=n_slots)
+    return lora_op(y1, x, kb, vb, a_start, a_len, a_loc, mrg_ids, slot, -scales, n_slots=n_slots)

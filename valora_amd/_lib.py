@@ -27,7 +27,7 @@ SYMBOLS = [
     "mlora_lora_apply_multi", "mlora_lora_fused", "mlora_dispatch_bgmv",
     "mlora_dispatch_sgmm", "mlora_prefill_shrink", "mlora_prefill_expand",
     "mlora_pool_alloc", "mlora_pool_alloc_contiguous", "mlora_pool_free", "mlora_pool_fill",
-    "mlora_pool_scatter_rows", "mlora_pool_gather_rows", "mlora_index_compact",
+    "mlora_pool_scatter_rows", "mlora_pool_gather_rows", "mlora_index_compact", "mlora_merge_adapter",
 ]
 
 
@@ -109,6 +109,8 @@ def lib():
     L.mlora_index_compact.argtypes = [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
                                       c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                       c_void_p]
+    L.mlora_merge_adapter.argtypes = [c_void_p, POINTER(c_void_p), POINTER(c_int32), c_int32, c_int64, c_int64, c_int64,
+                                      POINTER(Pool), POINTER(Pool), c_int64, c_int64, ctypes.c_float, c_int32, c_int]
     for n in SYMBOLS[5:]:  # everything after the size queries returns a status
         getattr(L, n).restype = c_int
     _lib = L
