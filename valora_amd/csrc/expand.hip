@@ -26,13 +26,6 @@ constexpr int STAGE_LD = EXP_WN + 4;
 constexpr int EXP_MBU = 2;         // 16-token blocks whose loads are in flight together
 constexpr int EXP_MAX_BM = 256;   // tallest expand tile (tokens), one thread per token at set-up
 
-#ifdef MLORA_TRACE
-__device__ long long g_trace_e[4096 * 8];
-#define TRACE_E(i) \
-  if (threadIdx.x == 0) g_trace_e[(blockIdx.y * gridDim.x + blockIdx.x) % 4096 * 8 + (i)] = wall_clock64()
-#else
-#define TRACE_E(i)
-#endif
 
 // the arguments of target z of a multi-target launch
 __device__ __forceinline__ ExpandArgs select_target(const ExpandArgs &a, int z) {
@@ -56,7 +49,6 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs args_in) {
 
   const int tile_idx = blockIdx.x / p.n_ochunks;
   const int oc = blockIdx.x - tile_idx * p.n_ochunks;
-  TRACE_E(0);
   const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int a = tile[0], r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
@@ -92,7 +84,6 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs args_in) {
     }
   }
   s_perm[tid] = my_perm;
-  TRACE_E(1);
   // The only workgroup-wide barrier: it also drains the loads above (which everything below needs
   // anyway).  No barrier may follow the bulk loads below -- a barrier waits for all outstanding
   // global loads and would serialise the B, y and v traffic into separate round trips.
@@ -109,7 +100,6 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs args_in) {
                                                         : u32x4{0, 0, 0, 0};
     }
 
-  TRACE_E(2);
   // row-major roles for the y read-modify-write: 8 lanes x 16 B cover one token row of the wave's
   // 64 outputs; a wave covers 8 rows per access, two accesses per 16-token block.
   const int rr0 = lane >> 3, c8 = (lane & 7) * 8;
@@ -204,18 +194,7 @@ __global__ __launch_bounds__(256) void expand_kernel(ExpandArgs args_in) {
         __builtin_amdgcn_wave_barrier();
       }
     }
-#ifdef MLORA_TRACE
-    if (mb0 == 0) TRACE_E(3);
-#endif
   }
-#ifdef MLORA_TRACE
-  __builtin_amdgcn_s_waitcnt(0);
-  TRACE_E(4);
-  if (threadIdx.x == 0) {
-    long long *tr = g_trace_e + (blockIdx.y * gridDim.x + blockIdx.x) % 4096 * 8;
-    tr[5] = cnt; tr[6] = tile_idx; tr[7] = oc;
-  }
-#endif
 }
 
 template <typename T>
@@ -254,9 +233,3 @@ int launch_expand(hipStream_t st, const ExpandArgs &a, int max_rank, int64_t gri
 int expand_bn() { return EXP_BN; }
 
 }  // namespace mlora
-
-#ifdef MLORA_TRACE
-extern "C" int mlora_dbg_trace_e(long long *out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(mlora::g_trace_e), sizeof(long long) * 4096 * 8);
-}
-#endif

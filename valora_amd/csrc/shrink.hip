@@ -20,14 +20,6 @@ namespace mlora {
 
 namespace {
 
-#ifdef MLORA_TRACE
-__device__ long long g_trace[4096 * 8];
-#define TRACE_T(i)                                                                                              \
-  if (threadIdx.x == 0)                                                                                         \
-  g_trace[((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) % 4096 * 8 + (i)] = wall_clock64()
-#else
-#define TRACE_T(i)
-#endif
 
 // the arguments of target z of a multi-target launch
 __device__ __forceinline__ ShrinkArgs select_target(const ShrinkArgs &a, int z) {
@@ -277,7 +269,6 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
   constexpr int RING_BYTES = STAGES * STAGE_BYTES + 1024;   // + one scratch block for dummy loads
   __shared__ __align__(16) unsigned char s_raw[RING_BYTES > TILE_BYTES ? RING_BYTES : TILE_BYTES];
 
-  TRACE_T(0);
   const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
@@ -352,11 +343,7 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
 #pragma unroll
     for (int i = 0; i < APW; ++i) {
       unsigned char *dst = sbase + a_off + (wave * APW + i) * 1024;
-#ifdef MLORA_EXP_NOA
-      load_or_dummy(false, ap[i] + kbeg + step * KC, dst);
-#else
       load_or_dummy(aok[i] && kok, ap[i] + kbeg + step * KC, dst);
-#endif
       if (!kok) lds_write16(lds_offset(dst) + lane * 16, zero4);
     }
   };
@@ -371,7 +358,6 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  TRACE_T(1);
   issue(0);
   if (n_steps > 1) issue(1);
   for (int step = 0; step < n_steps; ++step) {
@@ -380,17 +366,10 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
     // iteration is free to be refilled
     if (step + 1 < n_steps) wait_vmcnt<LOADS_PER_STAGE>(); else wait_vmcnt<0>();
     wait_lgkmcnt0();
-#ifndef MLORA_EXP_NOBARRIER
     __builtin_amdgcn_s_barrier();
-#endif
-    if (step == 0) TRACE_T(4);
     if (step + 2 < n_steps) issue(step + 2);
     const int stage = step % STAGES;
-#ifdef MLORA_EXP_NOCOMPUTE
-    if (false) {
-#else
     if (wave_active) {
-#endif
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         u32x4 xf[MBW], bf[NB];
@@ -417,7 +396,6 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
     }
   }
   wait_lgkmcnt0();
-  TRACE_T(2);
   __syncthreads();   // everybody is done reading the ring: reuse it for the result tile
 
   float *otile = reinterpret_cast<float *>(s_raw);
@@ -433,16 +411,6 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
       }
   __syncthreads();
   shrink_epilogue<T>(p, otile, NB * 16, s, pos0, cnt, r, perm);
-#ifdef MLORA_TRACE
-  __builtin_amdgcn_s_waitcnt(0);
-  TRACE_T(3);
-  if (threadIdx.x == 0) {
-    long long *tr = g_trace + ((blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) % 4096 * 8;
-    tr[5] = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (3 << 11)) /* XCC_ID */;
-    tr[6] = n_steps;
-    tr[7] = tile_idx * 100 + s;
-  }
-#endif
 }
 
 template <typename T>
@@ -507,9 +475,3 @@ int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int
 }
 
 }  // namespace mlora
-
-#ifdef MLORA_TRACE
-extern "C" void mlora_dbg_trace(long long *out) {
-  hipMemcpyFromSymbol(out, HIP_SYMBOL(mlora::g_trace), sizeof(long long) * 4096 * 8);
-}
-#endif
