@@ -213,8 +213,80 @@ def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0):
         torch.cuda.empty_cache()
     if not only:
         report["adapter_residency"] = bench_adapter_residency(torch, dev)
+        report["config5_step"] = bench_config5_step(torch, W, dev, use_graph)
     with open(path, "w") as f:
         json.dump(report, f, indent=1)
+
+
+def bench_config5_step(torch, W, dev, use_graph):
+    """The serving step of benchmark configuration 5: 32 decoder layers of the 7B shape (hidden 4096, 32 heads,
+    MLP 11008, random weights), 128 decode tokens with cached contexts of 256..2048 tokens plus 2 prefill
+    requests of 512 tokens, 64 resident adapters (ranks 16/32/64, Zipf 0.8), LoRA on all 7 projections.  The base
+    model is stock PyTorch (mm, scaled_dot_product_attention); reported: step time with LoRA, base-only step time
+    and their difference.  The KV cache is shared by the layers (it only serves the timing of the base step)."""
+    import torch.nn.functional as F
+    from valora_amd.layer import LayerPlans, LayerPools, LayerWeights, layer_forward
+    H, MLP, heads, L, dt = 4096, 11008, 32, 32, torch.bfloat16
+    d = H // heads
+    w5 = W.CONFIGS[5]()
+    wd = w5.to(dev)
+    T, n_dec = w5.T, 128
+    pa, pu, pdn = wd.target("q").pool, wd.target("gate").pool, wd.target("down").pool
+    idx = (pa.a_start, pa.a_len, pa.a_loc, pa.a_scaling)
+    g = torch.Generator(device=dev).manual_seed(55)
+    rnd = lambda *shape, s=1.0: (torch.randn(*shape, device=dev, generator=g) * s).to(dt)
+    layers = []
+    for _ in range(L):
+        wts = LayerWeights(rnd(H, H, s=H ** -0.5), rnd(H, H, s=H ** -0.5), rnd(H, H, s=H ** -0.5), rnd(H, H, s=H ** -0.5),
+                           rnd(H, MLP, s=H ** -0.5), rnd(H, MLP, s=H ** -0.5), rnd(MLP, H, s=MLP ** -0.5),
+                           torch.ones(H, device=dev, dtype=dt), torch.ones(H, device=dev, dtype=dt))
+        pools = LayerPools(tuple(rnd(*b.shape, s=0.02) for b in (pa.key_buffer, pa.value_buffer)),
+                           tuple(rnd(*b.shape, s=0.02) for b in (pu.key_buffer, pu.value_buffer)),
+                           tuple(rnd(*b.shape, s=0.02) for b in (pdn.key_buffer, pdn.value_buffer)), *idx)
+        layers.append((wts, pools))
+    plans = LayerPlans(wd.ids, pa.a_start, pa.a_len, max(pa.ranks), H, MLP)
+    gl = torch.Generator().manual_seed(56)
+    kv_len = torch.randint(256, 2049, (n_dec,), generator=gl)
+    Lmax = int(kv_len.max())
+    kc, vc = rnd(n_dec, heads, Lmax, d), rnd(n_dec, heads, Lmax, d)
+    mask = (torch.arange(Lmax)[None, :] < kv_len[:, None]).to(dev)[:, None, None, :]
+    pre = [(n_dec + i * 512, n_dec + (i + 1) * 512) for i in range(2)]
+
+    def attention(q, k, v):
+        out = torch.empty_like(q)
+        out[:n_dec] = F.scaled_dot_product_attention(q[:n_dec].view(n_dec, heads, 1, d), kc, vc,
+                                                     attn_mask=mask).reshape(n_dec, H)
+        for b, e in pre:
+            qq, kk, vv = (t[b:e].view(512, heads, d).transpose(0, 1).unsqueeze(0) for t in (q, k, v))
+            out[b:e] = F.scaled_dot_product_attention(qq, kk, vv, is_causal=True)[0].transpose(0, 1).reshape(512, H)
+        return out
+
+    pos = torch.cat((kv_len.float(), torch.arange(512).float(), torch.arange(512).float())).to(dev)
+    freq = 1.0 / (10000 ** (torch.arange(0, d, 2, device=dev).float() / d))
+    ang = torch.cat((pos[:, None] * freq[None], pos[:, None] * freq[None]), dim=-1)
+    cos, sin = ang.cos().to(dt), ang.sin().to(dt)
+    x0 = rnd(T, H)
+
+    def step(lora):
+        x = x0
+        for wts, pools in layers:
+            x = layer_forward(x, wts, pools if lora else None, plans if lora else None, attention, heads, cos, sin)
+        return x
+
+    out = {}
+    for name, lora in (("base_only", False), ("with_lora", True)):
+        try:
+            ms, _ = time_graph(torch, lambda: step(lora), 5, 2, use_graph)
+            mode = "hip graph replay" if use_graph else "eager"
+        except Exception as exc:   # a library call that cannot be captured: time it eagerly
+            torch.cuda.synchronize()
+            ms, _ = time_graph(torch, lambda: step(lora), 5, 2, False)
+            mode = f"eager ({type(exc).__name__} during capture)"
+        out[name] = {"ms_per_step": round(ms, 3), "launch": mode}
+    out["lora_overhead_ms"] = round(out["with_lora"]["ms_per_step"] - out["base_only"]["ms_per_step"], 3)
+    out["tokens"] = T
+    out["lora_calls_per_layer"] = 4
+    return out
 
 
 def bench_adapter_residency(torch, dev):
