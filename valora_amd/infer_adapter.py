@@ -341,6 +341,10 @@ class InferAdapter:
         if len(reserve_adapter_dirs) == len(self.adapter_dirs):
             return
         dev = self.mem_manager.device
+        if self.prefetch_stream is not None:
+            # rows freed below may be handed out again at once: copies still running on the prefetch stream
+            # must have landed first
+            torch.cuda.current_stream(dev).wait_stream(self.prefetch_stream)
         if len(reserve_adapter_dirs) == 0:
             self.mem_manager.free(self.a_loc)
             self.adapter_dirs = []
