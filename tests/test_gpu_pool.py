@@ -231,6 +231,22 @@ def test_infer_adapter_random_history_vs_oracle(dev):
         assert_same_residency(ia, res)
 
 
+def test_offload_everything_by_naming_no_resident_adapter(dev):
+    """A reserve list that names nobody resident drops every adapter (the reference's tensor code indexes
+    an empty tensor in this case); rows, index and counters end up as after a full offload."""
+    spec = {f"e{i}": dict(r=2, scaling=1.0) for i in range(3)}
+    prod, _ = weights_from_oracle_spec(spec, 4)
+    heads, H, L = NET["num_attention_heads"], NET["hidden_size"], NET["num_hidden_layers"]
+    mm = MemoryAllocator(40, 40, torch.float16, heads, H // heads, L, dev)
+    ia = InferAdapter.init(mm)
+    ia.load_adapters(list(prod.values()))
+    ia.offload_adapters(["somebody-else"])
+    assert ia.adapter_dirs == [] and ia.idx_map == {} and ia.a_loc.numel() == 0 and ia.a_start.numel() == 0
+    assert mm.can_use_mem_size == 40 and bool(mm.mem_state.all())
+    ia.load_adapters([prod["e1"]])
+    assert ia.a_loc.tolist() == list(range(8)) and ia.a_start.tolist() == [0]
+
+
 def test_contiguous_rows_option(dev):
     spec = {f"c{i}": dict(r=2, scaling=1.0) for i in range(5)}
     prod, _ = weights_from_oracle_spec(spec, 4)
