@@ -14,17 +14,18 @@
 // B of a slot is [H_out, r] flat over r pool rows -- K-contiguous for the MFMA, loaded straight
 // into registers as in the expand.  A of a slot is r pool rows of H_in elements, i.e. [r, H_in]:
 // the MFMA wants 8 consecutive rank elements of ONE input row per lane, so the workgroup's
-// [r x 128] slice of A goes through LDS and is read back transposed with 2-byte reads (the row
-// stride of 132 elements spreads the four rank groups of a wave over different banks).
+// [r x tile height] slice of A goes through LDS and is read back transposed with 2-byte reads (the row
+// stride of tile height + 4 elements spreads the four rank groups of a wave over different banks).
 #include "kernel_common.h"
 
 namespace mlora {
 
 namespace {
 
-constexpr int MG_BM = 128;        // input rows (of W) per workgroup
 constexpr int MG_BN = 256;        // output columns per workgroup, 64 per wave
-constexpr int MG_RS = 132;        // LDS row stride of the A slice, elements
+// input rows (of W) per workgroup: taller tiles re-read B less often, but the transposed LDS reads of the
+// A slice grow with the rank -- 256 rows measured faster up to rank 32, 128 rows above
+constexpr int merge_bm(int kb) { return kb == 1 ? 256 : 128; }
 constexpr int MG_STAGE_LD = 64 + 4;
 
 struct MergeArgs {
@@ -43,6 +44,8 @@ template <typename T, int KB>
 __global__ __launch_bounds__(256) void merge_kernel(MergeArgs p) {
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
+  constexpr int MG_BM = merge_bm(KB);
+  constexpr int MG_RS = MG_BM + 4;   // LDS row stride of the A slice, elements (see the file header)
   __shared__ __align__(16) uint16_t s_a[KB * 32][MG_RS];
   __shared__ float stage[4][16][MG_STAGE_LD];
 
@@ -94,7 +97,7 @@ __global__ __launch_bounds__(256) void merge_kernel(MergeArgs p) {
     }
   }
 
-  // ---- the [r x 128] slice of A into LDS (rank rows beyond r are zero)
+  // ---- the [r x MG_BM] slice of A into LDS (rank rows beyond r are zero)
   for (int idx = tid; idx < KB * 32 * (MG_BM / 8); idx += 256) {
     const int j = idx / (MG_BM / 8), c = idx - j * (MG_BM / 8);
     const int i = i0 + c * 8;
@@ -236,7 +239,8 @@ extern "C" int mlora_merge_adapter(void *stream, void *const *w, const int32_t *
   a.n_ochunks = (int)((h_out + MG_BN - 1) / MG_BN);
   int kb = (int)((max_rank + 31) / 32);
   kb = kb <= 1 ? 1 : kb <= 2 ? 2 : 4;
-  const int64_t blocks = ((h_in + MG_BM - 1) / MG_BM) * a.n_ochunks;
+  const int bm = merge_bm(kb);
+  const int64_t blocks = ((h_in + bm - 1) / bm) * a.n_ochunks;
   dim3 grid((unsigned)blocks, (unsigned)n_targets);
   return dtype == MLORA_F16 ? launch_merge_t<_Float16>((hipStream_t)stream, a, kb, grid)
                             : launch_merge_t<__bf16>((hipStream_t)stream, a, kb, grid);
