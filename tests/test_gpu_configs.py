@@ -204,3 +204,33 @@ def test_full_size_properties(dev, n):
         assert torch.equal(part[::3], y0[::3])
         keep = torch.ones(w.T, dtype=torch.bool, device=dev); keep[::3] = False
         assert torch.equal(part[keep], base[keep])
+
+
+@pytest.mark.parametrize("dtype,T,hidden,h_out", [(torch.bfloat16, 150_000, 4096, 4096), (torch.float16, 70_000, 4096, 11008)])
+def test_very_large_batches_sampled_rows(dev, dtype, T, hidden, h_out):
+    """Batches far past the benchmark sizes (element offsets beyond 2^31 bytes): every token's result depends
+    on that token alone, so a sample of rows is checked against the oracle run on just those rows."""
+    from valora_amd.plan import LoraPlan
+    g = torch.Generator().manual_seed(T)
+    ranks = [16, 64, 32, 8, 64, 16, 32, 64]
+    pool = W.make_pool(ranks, hidden, h_out, dtype, g, True, scalings=[0.5, 1.0, 2.0, 1.0, 0.25, 1.0, 1.0, 2.0])
+    lens = torch.randint(1, 4000, (200,), generator=g)
+    lens = (lens.float() / lens.sum() * T).long().clamp_min(1)
+    lens[-1] += T - int(lens.sum())
+    req = torch.randint(-1, len(ranks), (200,), generator=g)
+    ids = torch.repeat_interleave(req, lens)
+    assert ids.numel() == T
+    pd = pool.to(dev)
+    x = torch.randn(T, hidden, device=dev, dtype=dtype)
+    y0 = torch.randn(T, h_out, device=dev, dtype=dtype)
+    y = y0.clone()
+    plan = LoraPlan(ids.to(dev), pd.a_start, pd.a_len, 64, hidden=hidden)
+    plan.apply(y, x, pd.key_buffer, pd.value_buffer, pd.a_start, pd.a_len, pd.a_loc, 1, pd.a_scaling)
+    rows = torch.cat((torch.tensor([0, 1, T - 2, T - 1]), torch.randint(0, T, (380,), generator=g)))
+    want = O.lora_op(y0[rows.to(dev)].cpu(), x[rows.to(dev)].cpu(), pool.key_buffer, pool.value_buffer, pool.a_start,
+                     pool.a_len, pool.a_loc, ids[rows], 1, pool.a_scaling)
+    assert_parity(y[rows.to(dev)].cpu(), want, f"T={T} sampled rows")
+    none = (ids < 0).to(dev)
+    assert torch.equal(y[none], y0[none])
+    changed = (y != y0).any(dim=1)
+    assert bool((changed == ~none).all()), "exactly the tokens with an adapter change"
