@@ -243,3 +243,49 @@ def test_edge_cases_empty_and_no_adapter(dev):
         plan16.apply_fused(yy, x2.to(dev), p2d.key_buffer, p2d.value_buffer, p2d.a_start, p2d.a_len, p2d.a_loc, slot,
                            p2d.a_scaling)
         assert_parity(yy.cpu(), want, f"fused n_slots={n_slots}")
+
+
+def test_plan_reuse_across_drop_in_calls(dev):
+    """The shims keep the plan of a batch while the caller keeps passing the same, unmodified tensors; a
+    modified or a different ids tensor gets a plan of its own."""
+    from valora_amd import _plan_cache
+    from valora_amd.kernels import dispatch_bgmv
+    w = W.config2(hidden=512, n_tokens=96, n_adapters=24)
+    wd = w.to(dev)
+    t = wd.target("q"); p = t.pool; pc = w.target("q").pool
+    R = max(p.ranks)
+
+    def run(ids_dev):
+        y = wd.y0["q"].clone()
+        delta = torch.zeros(wd.T, R, dtype=wd.dtype, device=dev)
+        dispatch_bgmv(delta, wd.x[t.h_in], p.key_buffer, p.a_start, p.a_len, p.a_loc, ids_dev, t.slot, p.a_scaling)
+        dispatch_bgmv(y, delta, p.value_buffer, p.a_start, p.a_len, p.a_loc, ids_dev, t.slot, p.a_scaling)
+        return y.cpu()
+
+    def want(ids_cpu):
+        return O.lora_op(w.y0["q"], w.x[t.h_in], pc.key_buffer, pc.value_buffer, pc.a_start, pc.a_len, pc.a_loc,
+                         ids_cpu, t.slot, pc.a_scaling)
+
+    _plan_cache.clear()
+    h0, m0 = _plan_cache.hits, _plan_cache.misses
+    ids = wd.ids.clone()
+    assert_parity(run(ids), want(w.ids), "first call")
+    assert_parity(run(ids), want(w.ids), "second call")
+    assert _plan_cache.misses - m0 == 1 and _plan_cache.hits - h0 == 3          # one build for four calls
+    # modified in place: the version counter moves, the old plan must not be used
+    ids2_cpu = (w.ids + 1) % 24
+    ids.copy_(ids2_cpu)
+    assert_parity(run(ids), want(ids2_cpu), "after an in-place change of the ids")
+    assert _plan_cache.misses - m0 == 2
+    # a different tensor object with other contents
+    ids3_cpu = torch.flip(w.ids, dims=(0,)).contiguous()
+    assert_parity(run(ids3_cpu.to(dev)), want(ids3_cpu), "new ids tensor")
+    assert _plan_cache.misses - m0 == 3
+    # switched off: same results, nothing cached
+    _plan_cache.set_enabled(False)
+    try:
+        h1, m1 = _plan_cache.hits, _plan_cache.misses
+        assert_parity(run(ids), want(ids2_cpu), "cache disabled")
+        assert (_plan_cache.hits, _plan_cache.misses) == (h1, m1)
+    finally:
+        _plan_cache.set_enabled(True)

@@ -1,0 +1,59 @@
+"""Reuse of the per-batch plan by the drop-in entry points.
+
+The reference's entry points take the per-token adapter ids with every call, and its caller passes
+the SAME tensors for all 8 calls of a layer and for all layers of a forward pass
+(valora/models/peft/lora_unordered_batch_infer.py:946-1063: ``self.batch_req_bins``,
+``self.infer_adapter.a_start / a_len``).  Sorting the tokens and cutting tiles once per call would cost
+more than the op itself at decode sizes, so the shims keep the plans of the last few distinct
+argument sets.  An entry is reused only if the call passes the very same tensor objects (weak
+references, so a new tensor at a recycled address never matches) and none of them has been modified
+in place through PyTorch since (``Tensor._version``).  Writes that bypass PyTorch's bookkeeping (a
+foreign kernel given the raw pointer) are not seen: ``set_enabled(False)`` turns the reuse off.
+"""
+from __future__ import annotations
+
+import weakref
+from typing import Callable, List, Sequence, Tuple
+
+import torch
+
+_MAX_ENTRIES = 8
+_enabled = True
+_entries: List[tuple] = []      # (weakrefs, versions, scalars, value), most recent last
+hits = 0
+misses = 0
+
+
+def set_enabled(flag: bool) -> None:
+    global _enabled
+    _enabled = bool(flag)
+    if not _enabled:
+        clear()
+
+
+def enabled() -> bool:
+    return _enabled
+
+
+def clear() -> None:
+    _entries.clear()
+
+
+def lookup(tensors: Sequence[torch.Tensor], scalars: Tuple, build: Callable[[], object]):
+    """The value built for exactly these tensor objects (unmodified since) and scalars, or a new one."""
+    global hits, misses
+    versions = tuple(t._version for t in tensors)
+    for i in range(len(_entries) - 1, -1, -1):
+        refs, vers, sc, value = _entries[i]
+        if sc == scalars and vers == versions and all(r() is t for r, t in zip(refs, tensors)):
+            if i != len(_entries) - 1:
+                _entries.append(_entries.pop(i))
+            hits += 1
+            return value
+    misses += 1
+    value = build()
+    _entries.append((tuple(weakref.ref(t) for t in tensors), versions, scalars, value))
+    # drop entries whose tensors are gone, then the oldest
+    _entries[:] = [e for e in _entries if all(r() is not None for r in e[0])]
+    del _entries[:-_MAX_ENTRIES]
+    return value

@@ -19,7 +19,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from .kernels import _check_common, _no_kernel, _workspace
+from .kernels import _cached_plan, _check_common, _no_kernel, _planned_call, _workspace
 
 _SHRINK_MODE = _lib.SHRINK_OVERWRITE
 
@@ -48,6 +48,21 @@ def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, q
     if lora_scales is not None and lora_scales.dtype != x.dtype:
         lora_scales = lora_scales.to(x.dtype)
     pool = _lib.make_pool(w, start_indicies, lora_ranks, loc_indicies, max(h_in, h_out), 4)
+    narrow = min(h_in, h_out)
+    oc, st = output_counts.contiguous(), start_ids.contiguous()
+
+    def ids_of_segments():
+        eff = torch.empty(T, dtype=torch.long, device=x.device)
+        _lib.check(_lib.lib().mlora_ids_from_segments(_lib.current_stream(x.device), _lib.ptr(eff), _lib.ptr(indicies),
+                                                      _lib.ptr(st), _lib.ptr(oc), P, T))
+        return eff
+
+    plan = _cached_plan(indicies, start_indicies, lora_ranks, T, narrow, max(h_in, h_out),
+                        extra_tensors=(output_counts, start_ids), extra_scalars=(P,), make_ids=ids_of_segments)
+    if plan is not None:
+        _planned_call(plan, _lib.current_stream(x.device), y, x, pool, qkvo, lora_scales, T, h_in, h_out, code,
+                      shrink_mode=_SHRINK_MODE)
+        return
     need = int(_lib.lib().mlora_workspace_bytes(T, start_indicies.numel(), min(h_in, h_out)))
     if (tmp_d is not None and tmp_d.is_cuda and tmp_d.is_contiguous() and tmp_d.element_size() == 1
             and tmp_d.numel() >= need and tmp_d.data_ptr() % 16 == 0):

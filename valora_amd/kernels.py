@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from . import _lib
+from . import _lib, _plan_cache
 
 
 def _check_input(t: torch.Tensor, name: str) -> None:
@@ -67,7 +67,51 @@ def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, q
     if lora_scales is not None and lora_scales.dtype != x.dtype:
         lora_scales = lora_scales.to(x.dtype)  # the kernel reads scales as T (bgmv_impl.cuh:180)
     pool = _lib.make_pool(w, start_indicies, lora_ranks, loc_indicies, wide, 4)
-    ws = _workspace(T, start_indicies.numel(), min(h_in, h_out), x.device)
+    narrow = min(h_in, h_out)
+    plan = _cached_plan(indicies, start_indicies, lora_ranks, T, narrow, wide)
+    stream = _lib.current_stream(x.device)
+    if plan is not None:
+        _planned_call(plan, stream, y, x, pool, qkvo, lora_scales, T, h_in, h_out, code)
+        return
+    ws = _workspace(T, start_indicies.numel(), narrow, x.device)
     _lib.check(_lib.lib().mlora_dispatch_bgmv(
-        _lib.current_stream(x.device), _lib.ptr(y), _lib.ptr(x), pool, _lib.ptr(indicies), int(qkvo),
+        stream, _lib.ptr(y), _lib.ptr(x), pool, _lib.ptr(indicies), int(qkvo),
         _lib.ptr(lora_scales), T, h_in, h_out, code, _lib.ptr(ws), ws.numel()))
+
+
+def _planned_call(plan, stream, y, x, pool, qkvo, scales, T, h_in, h_out, code, shrink_mode=_lib.SHRINK_OVERWRITE,
+                  shrink_width=0, y_stride=None, x_stride=None) -> None:
+    """One shrink or one expand launch on a plan that already exists: the argument mapping of the one-call
+    entry points (direction by ``h_in < h_out``, valora/csrc/bgmv/bgmv_impl.cuh:221) minus the plan build."""
+    narrow = min(h_in, h_out)
+    if h_in < h_out:
+        if scales is None:
+            raise RuntimeError("lora_scales is null")
+        _lib.check(_lib.lib().mlora_expand(stream, plan.handle, _lib.ptr(y), T, h_out, None, _lib.ptr(x),
+                                           h_in if x_stride is None else x_stride, narrow, pool, int(qkvo),
+                                           _lib.ptr(scales), 1, 0, code))
+    else:
+        _lib.check(_lib.lib().mlora_shrink(stream, plan.handle, _lib.ptr(plan.scratch), plan.scratch.numel(),
+                                           _lib.ptr(x), T, h_in, narrow, pool, int(qkvo), int(plan.ksplit), _lib.ptr(y),
+                                           h_out if y_stride is None else y_stride, shrink_mode, shrink_width, 0, code))
+
+
+def _cached_plan(ids, a_start, a_len, T, narrow, wide, n_slots=4, extra_tensors=(), extra_scalars=(), make_ids=None):
+    """``make_ids``: builds the per-token ids the plan is cut from when the entry point does not get them
+    directly (segment or per-request operands); the result lives as long as the cache entry."""
+    """The plan of this batch from the cache (built on a miss), or None when the shapes are ones only
+    the one-call entry point reports properly (it raises the reference's errors)."""
+    if not _plan_cache.enabled() or T == 0 or narrow <= 0 or narrow > 128 or narrow % 8 or narrow >= wide:
+        return None
+    from .plan import LoraPlan
+    def build():
+        eff = ids if make_ids is None else make_ids()
+        plan = LoraPlan(eff, a_start, a_len, narrow, n_slots=n_slots, hidden=wide)
+        plan.ids_keepalive = eff
+        return plan
+
+    try:
+        return _plan_cache.lookup((ids, a_start, a_len) + tuple(extra_tensors),
+                                  (T, narrow, wide, n_slots, ids.device.index) + tuple(extra_scalars), build)
+    except RuntimeError:
+        return None
