@@ -47,6 +47,12 @@ __device__ __forceinline__ int block_exclusive_scan(int v, int *total, int *wsum
   return wsum[wave] + inc - v;
 }
 
+constexpr int PLAN_SMALL_A = 2048;   // adapters whose per-adapter tables fit in LDS next to the histograms
+
+// SMALL: the per-adapter tables (counts, group starts, tile offsets, ranks, a_start) live in LDS instead of
+// the plan's scratch area, so the dependent look-ups of the later phases (the binary search of the tile
+// lists above all) cost LDS latency instead of a global round trip each.
+template <bool SMALL>
 __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
     int32_t *__restrict__ plan, const int64_t *__restrict__ ids, const int64_t *__restrict__ a_start,
     const int64_t *__restrict__ a_len, int T, int A, int n_slots, int bm_s, int bm_e, int W,
@@ -57,17 +63,35 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
   __shared__ int s_maxrank;
   __shared__ int s_err;
 
+  __shared__ int32_t s_tab[SMALL ? 4 * PLAN_SMALL_A : 1];
+  __shared__ int32_t s_rank[SMALL ? PLAN_SMALL_A : 1];
+  __shared__ int64_t s_astart[SMALL ? PLAN_SMALL_A : 1];
+
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int32_t *perm = plan + off_perm;
   int32_t *padapter = plan + off_padapter;
   int32_t *prank = plan + off_prank;
-  int32_t *cnt = plan + off_scratch;
-  int32_t *gstart = cnt + A;
-  int32_t *toff_s = gstart + A;
-  int32_t *toff_e = toff_s + A;
+  int32_t *cnt = SMALL ? s_tab : plan + off_scratch;
+  int32_t *gstart = cnt + (SMALL ? PLAN_SMALL_A : A);
+  int32_t *toff_s = gstart + (SMALL ? PLAN_SMALL_A : A);
+  int32_t *toff_e = toff_s + (SMALL ? PLAN_SMALL_A : A);
+  // rank of adapter a (0 = not usable: ranks are multiples of 8 up to MAX_RANK) and its a_start
+  auto rank_of = [&](int a) -> int {
+    if (SMALL) return s_rank[a];
+    const int64_t r = a_len[a] / n_slots;
+    return (r > 0 && (r & 7) == 0 && r <= MAX_RANK) ? (int)r : 0;
+  };
+  auto start_of = [&](int a) -> int64_t { return SMALL ? s_astart[a] : a_start[a]; };
 
   for (int i = tid; i < W * A; i += PLAN_THREADS) whist[i] = 0;
   for (int i = tid; i < max_tiles; i += PLAN_THREADS) plan[off_counters + i] = 0;
+  if (SMALL) {
+    for (int a = tid; a < A; a += PLAN_THREADS) {
+      const int64_t r = a_len[a] / n_slots;
+      s_rank[a] = (r > 0 && (r & 7) == 0 && r <= MAX_RANK) ? (int)r : 0;
+      s_astart[a] = a_start[a];
+    }
+  }
   if (tid == 0) { s_maxrank = 0; s_err = 0; }
   __syncthreads();
 
@@ -76,13 +100,19 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
   const int t_beg = wave * cw;
   const int t_end = (wave < W) ? min(T, t_beg + cw) : 0;
 
-  // 1. per-wave histogram of valid tokens
+  // 1. per-wave histogram of valid tokens (the first 64 tokens of a wave stay in registers for step 3)
+  int first_a = -1, first_r = 0;
   for (int t = t_beg + lane; t < t_end; t += 64) {
-    const int64_t a = ids[t];
-    if (a >= 0 && a < A) {
-      const int64_t r = a_len[a] / n_slots;   // ranks are multiples of 8 (16-byte vectors)
-      if (r > 0 && (r & 7) == 0 && r <= MAX_RANK) atomicAdd(&whist[wave * A + (int)a], 1);
+    const int64_t a64 = ids[t];
+    int a = -1, r = 0;
+    if (a64 >= 0 && a64 < A) {
+      r = rank_of((int)a64);
+      if (r > 0) {
+        a = (int)a64;
+        atomicAdd(&whist[wave * A + a], 1);
+      }
     }
+    if (t < t_beg + 64) { first_a = a; first_r = r; }
   }
   __syncthreads();
 
@@ -99,7 +129,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
       my_ts += (c + bm_s - 1) / bm_s;
       my_te += (c + bm_e - 1) / bm_e;
       my_g += 1;
-      my_maxr = max(my_maxr, (int)(a_len[a] / n_slots));
+      my_maxr = max(my_maxr, rank_of(a));
     }
   }
   int n_active, n_ts, n_te, n_g;
@@ -130,11 +160,14 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
   for (int t0 = t_beg; t0 < t_end; t0 += 64) {
     const int t = t0 + lane;
     int a = -1, r = 0;
-    if (t < t_end) {
+    if (t0 == t_beg) {
+      a = first_a;
+      r = first_r;
+    } else if (t < t_end) {
       const int64_t a64 = ids[t];
       if (a64 >= 0 && a64 < A) {
-        r = (int)(a_len[a64] / n_slots);
-        if (r > 0 && (r & 7) == 0 && r <= MAX_RANK) a = (int)a64;
+        r = rank_of((int)a64);
+        if (r > 0) a = (int)a64;
       }
     }
     unsigned long long remaining = __ballot(a >= 0);
@@ -173,11 +206,11 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
       const int a = lo - 1;
       const int k = i - toff[a];
       const int c = cnt[a];
-      const int64_t st = a_start[a];
+      const int64_t st = start_of(a);
       if (st < 0 || st > 0x7fffffff) atomicOr(&s_err, (int)PERR_START_OVERFLOW);
       int32_t *tl = tiles + (int64_t)i * TILE_WORDS;
       tl[0] = a;
-      tl[1] = (int)(a_len[a] / n_slots);
+      tl[1] = rank_of(a);
       tl[2] = gstart[a] + k * bm;
       tl[3] = min(bm, c - k * bm);
       tl[4] = (int32_t)st;
@@ -280,9 +313,14 @@ int launch_plan(hipStream_t st, int32_t *plan, const PlanLayout &L, const int64_
   int W = A > 0 ? (int)(HIST_WORDS / A) : PLAN_WAVES;
   if (W > PLAN_WAVES) W = PLAN_WAVES;
   if (W < 1) return fail(MLORA_ERR_NO_KERNEL, "plan: more than %lld adapters", (long long)MAX_ADAPTERS);
-  hipLaunchKernelGGL(plan_kernel, dim3(1), dim3(PLAN_THREADS), 0, st, plan, ids, a_start, a_len,
-                     (int)L.T, A, n_slots, bm_s, bm_e, W, L.off_perm, L.off_padapter, L.off_prank,
-                     L.off_tiles_s, L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles);
+  if (A <= PLAN_SMALL_A)
+    hipLaunchKernelGGL(plan_kernel<true>, dim3(1), dim3(PLAN_THREADS), 0, st, plan, ids, a_start, a_len,
+                       (int)L.T, A, n_slots, bm_s, bm_e, W, L.off_perm, L.off_padapter, L.off_prank,
+                       L.off_tiles_s, L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles);
+  else
+    hipLaunchKernelGGL(plan_kernel<false>, dim3(1), dim3(PLAN_THREADS), 0, st, plan, ids, a_start, a_len,
+                       (int)L.T, A, n_slots, bm_s, bm_e, W, L.off_perm, L.off_padapter, L.off_prank,
+                       L.off_tiles_s, L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles);
   return check_launch("plan_kernel");
 }
 
