@@ -264,7 +264,8 @@ __global__ __launch_bounds__(256) void index_copy_loc_kernel(const int32_t *__re
                                                               int64_t *__restrict__ new_loc, int64_t new_loc_len) {
   const int a = keep[blockIdx.x];
   if (a < 0 || a >= n_old) return;
-  const int64_t len = old_len[a], src = old_start[a], dst = new_start[blockIdx.x];
+  const int64_t src = old_start[a], dst = new_start[blockIdx.x];
+  const int64_t len = min(old_len[a], old_loc_len);   // a corrupt length must not turn into a long loop
   for (int64_t j = threadIdx.x; j < len; j += 256)
     if (src + j >= 0 && src + j < old_loc_len && dst + j < new_loc_len) new_loc[dst + j] = old_loc[src + j];
 }
@@ -281,7 +282,8 @@ __global__ __launch_bounds__(256) void index_free_dropped_kernel(const int32_t *
   const int lo = g == 0 ? 0 : keep[g - 1] + 1;
   const int hi = g == n_keep ? n_old : keep[g];
   for (int a = max(lo, 0); a < min(hi, n_old); ++a) {
-    const int64_t len = old_len[a], src = old_start[a];
+    const int64_t src = old_start[a];
+    const int64_t len = min(old_len[a], old_loc_len);
     for (int64_t j = threadIdx.x; j < len; j += 256) {
       if (src + j < 0 || src + j >= old_loc_len) continue;
       const int64_t row = old_loc[src + j];
