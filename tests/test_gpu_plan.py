@@ -51,7 +51,7 @@ def _check_plan(ids_cpu, a_len_cpu, n_slots, bm_s, bm_e, dev):
 
 @pytest.mark.parametrize("T,A,style", [
     (1, 1, "random"), (256, 64, "zipf"), (1000, 7, "random"), (4416, 32, "runs"), (64, 600, "random"),
-    (5000, 5000, "random"), (300, 8192, "random"), (777, 3, "holes"), (20000, 16, "runs"), (0, 4, "random")])
+    (5000, 5000, "random"), (300, 8192, "random"), (3000, 2048, "random"), (3000, 2049, "random"), (777, 3, "holes"), (20000, 16, "runs"), (0, 4, "random")])
 def test_plan_invariants(dev, T, A, style):
     g = torch.Generator().manual_seed(T * 31 + A)
     a_len = torch.randint(1, 9, (A,), generator=g) * 8 * 4
