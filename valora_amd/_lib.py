@@ -136,7 +136,14 @@ def ptr(t) -> c_void_p:
     return c_void_p(0 if t is None else t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream(device) -> c_void_p:
+    """Handle of PyTorch's current stream on ``device`` (the raw getter saves ~4 us per call over building a
+    ``torch.cuda.Stream`` object; both name the same stream)."""
+    if _raw_stream is not None and device.index is not None:
+        return c_void_p(_raw_stream(device.index))
     return c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 

@@ -39,18 +39,25 @@ def clear() -> None:
     _entries.clear()
 
 
+def _same(refs, vers, tensors) -> bool:
+    for r, v, t in zip(refs, vers, tensors):
+        if r() is not t or v != t._version:
+            return False
+    return True
+
+
 def lookup(tensors: Sequence[torch.Tensor], scalars: Tuple, build: Callable[[], object]):
     """The value built for exactly these tensor objects (unmodified since) and scalars, or a new one."""
     global hits, misses
-    versions = tuple(t._version for t in tensors)
     for i in range(len(_entries) - 1, -1, -1):
         refs, vers, sc, value = _entries[i]
-        if sc == scalars and vers == versions and all(r() is t for r, t in zip(refs, tensors)):
+        if sc == scalars and _same(refs, vers, tensors):
             if i != len(_entries) - 1:
                 _entries.append(_entries.pop(i))
             hits += 1
             return value
     misses += 1
+    versions = tuple(t._version for t in tensors)
     value = build()
     _entries.append((tuple(weakref.ref(t) for t in tensors), versions, scalars, value))
     # drop entries whose tensors are gone, then the oldest

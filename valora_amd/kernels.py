@@ -20,10 +20,15 @@ def _check_input(t: torch.Tensor, name: str) -> None:
         raise RuntimeError(f"{name} must be contiguous")
 
 
+_NAMES = ("y", "x", "w", "start_indicies", "lora_ranks", "loc_indicies", "indicies")
+
+
 def _check_common(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies):
-    for t, n in ((y, "y"), (x, "x"), (w, "w"), (start_indicies, "start_indicies"),
-                 (lora_ranks, "lora_ranks"), (loc_indicies, "loc_indicies"), (indicies, "indicies")):
-        _check_input(t, n)
+    ts = (y, x, w, start_indicies, lora_ranks, loc_indicies, indicies)
+    for t in ts:
+        if not (t.is_cuda and t.is_contiguous()):     # the common case costs one pass; name the culprit below
+            for t2, n in zip(ts, _NAMES):
+                _check_input(t2, n)
     if y.dim() != 2:
         raise RuntimeError("y must be a 2D tensor")
     if x.dim() != 2:
@@ -36,10 +41,12 @@ def _check_common(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies):
         raise RuntimeError(f"CHECK_EQ(indicies.size(0), x.size(0)) failed. {indicies.size(0)} vs {x.size(0)}")
     if y.size(0) != x.size(0):
         raise RuntimeError(f"CHECK_EQ(y.size(0), x.size(0)) failed. {y.size(0)} vs {x.size(0)}")
-    for t, n in ((start_indicies, "start_indicies"), (lora_ranks, "lora_ranks"),
-                 (loc_indicies, "loc_indicies"), (indicies, "indicies")):
-        if t.dtype != torch.long:  # data_ptr<int64_t>() throws on any other type
-            raise RuntimeError(f"expected scalar type Long but found {t.dtype} ({n})")
+    long = torch.long
+    if not (start_indicies.dtype is long and lora_ranks.dtype is long and loc_indicies.dtype is long
+            and indicies.dtype is long):
+        for t, n in zip(ts[3:], _NAMES[3:]):
+            if t.dtype != torch.long:  # data_ptr<int64_t>() throws on any other type
+                raise RuntimeError(f"expected scalar type Long but found {t.dtype} ({n})")
 
 
 def _no_kernel(h_in, h_out, dtype):
@@ -97,14 +104,14 @@ def _planned_call(plan, stream, y, x, pool, qkvo, scales, T, h_in, h_out, code, 
 
 
 def _cached_plan(ids, a_start, a_len, T, narrow, wide, n_slots=4, extra_tensors=(), extra_scalars=(), make_ids=None):
-    """``make_ids``: builds the per-token ids the plan is cut from when the entry point does not get them
-    directly (segment or per-request operands); the result lives as long as the cache entry."""
     """The plan of this batch from the cache (built on a miss), or None when the shapes are ones only
-    the one-call entry point reports properly (it raises the reference's errors)."""
+    the one-call entry point reports properly (it raises the reference's errors).  ``make_ids`` builds the
+    per-token ids the plan is cut from when the entry point does not get them directly (segment or
+    per-request operands); the result lives as long as the cache entry."""
     if not _plan_cache.enabled() or T == 0 or narrow <= 0 or narrow > 128 or narrow % 8 or narrow >= wide:
         return None
-    from .plan import LoraPlan
     def build():
+        from .plan import LoraPlan
         eff = ids if make_ids is None else make_ids()
         plan = LoraPlan(eff, a_start, a_len, narrow, n_slots=n_slots, hidden=wide)
         plan.ids_keepalive = eff
