@@ -49,6 +49,9 @@ def parse():
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings with")
     ap.add_argument("--only-config", type=int, default=0,
                     help="with --all-configs: report this benchmark configuration only (1, 3, 4 or 5)")
+    ap.add_argument("--only-target", default=None,
+                    help="with --all-configs --only-config N: time this target only (q, k, v, o, gate, up, down) and "
+                         "no multi-target group, so that a profile of the run holds one shape per kernel")
     ap.add_argument("--all-configs", metavar="FILE", default=None,
                     help="also measure every target of configs 1,3,4,5 and write a JSON report to FILE")
     return ap.parse_args()
@@ -145,7 +148,7 @@ def cpu_baseline(torch, w, budget_s=15.0):
 COLD_BYTES = 1 << 30   # four times the 256 MB last-level cache of the MI355X
 
 
-def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0):
+def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0, only_target=None):
     """Per-target timing of the other benchmark configurations (report only; the JSON line of the
     default run is config 2).  Each target's shrink+expand is replayed back to back on 4 copies of y
     so that the read-modify-write does not hit the same lines (`us`: x and the pool may sit in the
@@ -158,6 +161,8 @@ def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0):
         rows = {}
         total_us = 0.0
         for t in wd.targets:
+            if only_target and t.name != only_target:
+                continue
             p = t.pool
             plan = LoraPlan(wd.ids, p.a_start, p.a_len, R, hidden=t.h_in)
             ycopies = [wd.y0[t.name].clone() for _ in range(4)]
@@ -202,7 +207,7 @@ def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0):
         groups, fused_total = {}, total_us
         for names in (("q", "k", "v"), ("gate", "up")):
             ts = [t for t in wd.targets if t.name in names]
-            if len(ts) < 2:
+            if len(ts) < 2 or only_target:
                 continue
             p = ts[0].pool
             plan = LoraPlan(wd.ids, p.a_start, p.a_len, R, hidden=ts[0].h_in)
@@ -496,7 +501,7 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, w)
     if args.all_configs:
-        bench_all_configs(torch, W, LoraPlan, dev, args.all_configs, use_graph, args.only_config)
+        bench_all_configs(torch, W, LoraPlan, dev, args.all_configs, use_graph, args.only_config, args.only_target)
     print(json.dumps(out))
 
 
