@@ -39,8 +39,13 @@ __device__ __forceinline__ ExpandArgs select_target(const ExpandArgs &a, int z) 
   return p;
 }
 
+// Waves per SIMD the register allocator has to leave room for.  The rank-64 variant that reads a finished
+// v sits 2 registers above the 96 that allow 5 waves; held to 5 it measured 1-6 % faster on the prefill and
+// mixed shapes (more workgroups resident per round), at 6 it spills.  The others are left to the compiler.
+constexpr int expand_min_waves(int kb, bool partial) { return (kb == 2 && !partial) ? 5 : 1; }
+
 template <typename T, int KB, bool PARTIAL>
-__global__ __launch_bounds__(256) void expand_kernel(ExpandArgs args_in) {
+__global__ __launch_bounds__(256, expand_min_waves(KB, PARTIAL)) void expand_kernel(ExpandArgs args_in) {
   const ExpandArgs p = select_target(args_in, blockIdx.y);
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
