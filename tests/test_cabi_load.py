@@ -94,3 +94,27 @@ def test_tile_table_lookup_and_fallback():
     fb = tt.fallback(300, 64, 4096, 200)            # decode-like -> direct 16-token tiles, expand sums the chunks
     assert fb.bm_shrink == 16 and fb.reduce_in_expand
     assert tt.key(300, 16, 4096, 64) == "1024:16:4096:128"
+
+
+def test_install_aliases_registers_the_reference_import_names():
+    import importlib
+    import sys
+    import types
+    import valora_amd
+    names = ("valora._kernels", "atmm_ops", "valora.models.peft.triton_kernel.lora.lora_prefill")
+    saved = {n: sys.modules.pop(n, None) for n in names}
+    try:
+        valora_amd.install_aliases()
+        assert importlib.import_module("atmm_ops").dispatch_bgmv is valora_amd.atmm_ops.dispatch_bgmv
+        assert sys.modules["valora._kernels"].dispatch_bgmv is valora_amd.kernels.dispatch_bgmv
+        m = sys.modules["valora.models.peft.triton_kernel.lora.lora_prefill"]
+        assert m.lora_get_qkvo_fwd_shrink is valora_amd.lora_prefill.lora_get_qkvo_fwd_shrink
+        valora_amd.install_aliases()                      # idempotent
+        sys.modules["atmm_ops"] = types.ModuleType("atmm_ops")
+        with pytest.raises(RuntimeError, match="already imported"):
+            valora_amd.install_aliases()
+    finally:
+        for n, m in saved.items():
+            sys.modules.pop(n, None)
+            if m is not None:
+                sys.modules[n] = m
