@@ -156,6 +156,42 @@ class LoraAdapterWeights:
         return cls(lora_dir, r, lora_alpha, network_config, packed)
 
     @classmethod
+    def from_hf_weights(cls, lora_dir: str, weights: Dict[str, torch.Tensor], lora_config: Dict,
+                        network_config: Dict[str, int], module_names: Sequence[str] = ("c_attn", "w1", "w2", "c_proj"),
+                        dtype=torch.float16, pin: bool = True) -> "LoraAdapterWeights":
+        """From a PEFT checkpoint's tensor dict, with the key scheme and the slicing of the reference's loader
+        (valora/models/peft/layer_weights/lora_layer_weight.py:434-516): the key prefix is the first key up to
+        ``layers``; layer ``l`` slot ``s`` reads ``{prefix}layers.{l}.self_attn.{module_names[s]}.lora_A.weight``
+        (``[r, >=H]``, its first H columns are kept) and ``...lora_B.weight`` (``[>=H, r]``, its first H rows are
+        kept -- the reference cuts a fused qkv or an MLP projection down to H the same way); a missing module is
+        zeros.  ``module_names`` defaults to the reference's Qwen names; pass e.g.
+        ``("q_proj", "k_proj", "v_proj", "o_proj")`` for Llama-style checkpoints."""
+        if not weights:
+            raise RuntimeError("empty adapter checkpoint")
+        r, alpha = int(lora_config["r"]), float(lora_config["lora_alpha"])
+        L, H = network_config["num_hidden_layers"], network_config["hidden_size"]
+        first = next(iter(weights.keys()))
+        cut = first.find("layers")
+        if cut < 0:
+            raise RuntimeError(f"cannot find 'layers' in checkpoint key {first!r}")
+        lora_A, lora_B = [], []
+        for l in range(L):
+            prefix = first[:cut] + f"layers.{l}.self_attn"
+            a_row, b_row = [], []
+            for m in module_names:
+                a = weights.get(f"{prefix}.{m}.lora_A.weight")
+                b = weights.get(f"{prefix}.{m}.lora_B.weight")
+                if a is not None and (a.dim() != 2 or a.shape[0] != r or a.shape[1] < H):
+                    raise RuntimeError(f"{prefix}.{m}.lora_A.weight has shape {tuple(a.shape)}, expected [{r}, >={H}]")
+                if b is not None and (b.dim() != 2 or b.shape[1] != r or b.shape[0] < H):
+                    raise RuntimeError(f"{prefix}.{m}.lora_B.weight has shape {tuple(b.shape)}, expected [>={H}, {r}]")
+                a_row.append(None if a is None else a[:, :H])
+                b_row.append(None if b is None else b[:H, :])
+            lora_A.append(a_row)
+            lora_B.append(b_row)
+        return cls.from_dense(lora_dir, r, alpha, network_config, lora_A, lora_B, dtype=dtype, pin=pin)
+
+    @classmethod
     def dummy(cls, lora_dir: str, r: int, lora_alpha: float, network_config: Dict[str, int], n_slots: int = 4,
               dtype=torch.float16, seed: int = 0, pin: bool = True) -> "LoraAdapterWeights":
         """Uniform(-1e-3, 1e-3) weights, the reference's dummy adapters (lora_layer_weight.py:311-331)."""
