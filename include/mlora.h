@@ -87,7 +87,7 @@ size_t mlora_workspace_bytes(int64_t T, int64_t n_adapters, int64_t max_rank);
  * [0, n_adapters) or an adapter of rank 0 marks a token that gets no LoRA).  Stable counting
  * sort of the tokens by adapter + one tile list per tile height.  Replaces the host-side
  * grouping done by precompute_sgmm_args_* (atmm/valora/csrc/bgmv/bgmv_impl.cuh:76-125).
- * bm_shrink, bm_expand: tile heights in tokens (16, 32 or 64 / any multiple of 16 up to 256);
+ * bm_shrink, bm_expand: tile heights in tokens (16, 32, 64 or 128 / any multiple of 16 up to 256);
  * 0 lets the library choose.                                                                 */
 int mlora_build_plan(void *stream, mlora_plan *plan, const int64_t *ids, int64_t T,
                      const int64_t *a_start, const int64_t *a_len, int64_t n_adapters,
