@@ -94,6 +94,12 @@ def test_tile_table_lookup_and_fallback():
     fb = tt.fallback(300, 64, 4096, 200)            # decode-like -> direct 16-token tiles, expand sums the chunks
     assert fb.bm_shrink == 16 and fb.reduce_in_expand
     assert tt.key(300, 16, 4096, 64) == "1024:16:4096:128"
+    assert tt.key(300, 24, 4096, 64) == "1024:32:4096:128" and tt.key(1, 8, 4096, 1) == "8:16:4096:1"
+    for rank in (8, 40, 128):                       # every table entry is a configuration the kernels take
+        for T in (1, 300, 5000, 100000):
+            c = tt.lookup(T, rank, 4096, 16)
+            assert c.bm_shrink in (16, 32, 64, 128) and not (rank > 64 and c.bm_shrink == 64)
+            assert 1 <= c.ksplit <= 64 and c.bm_expand % 16 == 0 and 16 <= c.bm_expand <= 256
 
 
 def test_install_aliases_registers_the_reference_import_names():

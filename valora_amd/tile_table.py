@@ -4,14 +4,16 @@ Replaces the reference's ``shape_to_config`` dictionary and ``get_config_a`` / `
 (valora/models/peft/lora_unordered_batch_infer.py:25-172,216-236), which map
 ``(n_adapters, first_seq_len, K, N)`` to CUTLASS threadblock / warp shapes tuned on an A100 and
 fall back to a fixed shape for unknown keys.  Here the key is
-``(token bucket, max rank, hidden, adapter bucket)`` and the value is what the HIP kernels can
-vary: the token height of a shrink tile, the split-K factor of the shrink and the token height
-of an expand tile.  Entries come from sweeps on MI355X (``tile_table.json`` next to this file);
-unknown keys fall back to a rule, like the reference's fallback tuple.
+``(token bucket, rank bucket, hidden, adapter bucket)`` and the value is what the HIP kernels can
+vary: the token height of a shrink tile, the split-K factor of the shrink, who sums the split-K
+chunks and the token height of an expand tile.  Entries come from sweeps on MI355X (``tile_table.json`` next to this file);
+a width without entries uses those of the nearest measured width, and anything else falls back to a
+rule, like the reference's fallback tuple.
 """
 from __future__ import annotations
 
 import json
+import math
 import os
 from dataclasses import dataclass
 from typing import Dict, Tuple
@@ -19,8 +21,9 @@ from typing import Dict, Tuple
 _HERE = os.path.dirname(os.path.abspath(__file__))
 TABLE_PATH = os.path.join(_HERE, "tile_table.json")
 
-TOKEN_BUCKETS = (64, 256, 1024, 4096, 16384, 1 << 22)
+TOKEN_BUCKETS = (8, 64, 256, 1024, 4096, 16384, 1 << 22)
 ADAPTER_BUCKETS = (1, 8, 32, 128, 8192)
+RANK_BUCKETS = (16, 32, 64, 128)
 
 
 @dataclass(frozen=True)
@@ -39,7 +42,8 @@ def _bucket(v: int, buckets) -> int:
 
 
 def key(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> str:
-    return f"{_bucket(n_tokens, TOKEN_BUCKETS)}:{max_rank}:{hidden}:{_bucket(n_adapters, ADAPTER_BUCKETS)}"
+    return (f"{_bucket(n_tokens, TOKEN_BUCKETS)}:{_bucket(max_rank, RANK_BUCKETS)}:{hidden}:"
+            f"{_bucket(n_adapters, ADAPTER_BUCKETS)}")
 
 
 def fallback(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> TileConfig:
@@ -55,6 +59,7 @@ def fallback(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> Tile
 
 
 _table: Dict[str, TileConfig] = {}
+_hiddens: list = []      # the widths the table has entries for
 _loaded = False
 
 
@@ -67,14 +72,23 @@ def _load() -> None:
         for k, v in raw.get("entries", {}).items():
             _table[k] = TileConfig(int(v["bm_shrink"]), int(v["ksplit"]), int(v["bm_expand"]),
                                    bool(v.get("reduce_in_expand", False)))
+        _hiddens[:] = sorted({int(k.split(":")[2]) for k in _table})
 
 
 def lookup(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> TileConfig:
     if not _loaded:
         _load()
     cfg = _table.get(key(n_tokens, max_rank, hidden, n_adapters))
+    if cfg is None and _hiddens:
+        # a width the table was not measured for: the entry of the nearest measured width (ratio-wise),
+        # with the split-K factor cut to what the width can be split into
+        near = min(_hiddens, key=lambda h: abs(math.log(h / max(1, hidden))))
+        cfg = _table.get(key(n_tokens, max_rank, near, n_adapters))
+        if cfg is not None:
+            cfg = TileConfig(cfg.bm_shrink, max(1, min(cfg.ksplit, hidden // 128)), cfg.bm_expand,
+                             cfg.reduce_in_expand and min(cfg.ksplit, hidden // 128) > 1)
     if cfg is None:
         return fallback(n_tokens, max_rank, hidden, n_adapters)
-    if max_rank > 64 and cfg.bm_shrink > 32:
+    if max_rank > 64 and cfg.bm_shrink == 64:     # ranks above 64 have no 64-token shrink tile
         cfg = TileConfig(32, cfg.ksplit, cfg.bm_expand, cfg.reduce_in_expand)
     return cfg
