@@ -117,3 +117,27 @@ def test_random_shape_drop_in_bgmv(dev, seed):
     want = O.bgmv_expand(y0, delta.cpu(), pool.value_buffer, *cidx, ids, slot, pool.a_scaling)
     assert_parity(y.cpu(), want, what + " expand")
     assert torch.equal(y.cpu()[ids < 0], y0[ids < 0]), what
+
+
+@pytest.mark.parametrize("bm_shrink", [16, 32, 128])
+@pytest.mark.parametrize("ksplit,h_in", [(16, 4096), (32, 4096), (32, 11008), (64, 1032), (64, 8192)])
+def test_many_k_chunks(dev, bm_shrink, ksplit, h_in):
+    """Split-K counts the tile table uses for small batches and wide inputs, including more chunks than the
+    width has 128-element pieces (the surplus chunks are empty and must contribute zeros), with both ways
+    of summing the chunks."""
+    g = torch.Generator().manual_seed(ksplit + h_in)
+    ranks, T, h_out = [64, 16, 128, 8], 70, 520
+    pool = W.make_pool(ranks, h_in, h_out, torch.bfloat16, g, True, std=0.05, scalings=[1.0, 0.5, 2.0, 0.25], heads=1)
+    ids = torch.randint(-1, len(ranks), (T,), generator=g)
+    x = torch.randn(T, h_in, generator=g).bfloat16()
+    y0 = torch.randn(T, h_out, generator=g).bfloat16()
+    want = O.lora_op(y0, x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, 2,
+                     pool.a_scaling)
+    pd = pool.to(dev)
+    for rie in (False, True):
+        plan = LoraPlan(ids.to(dev), pd.a_start, pd.a_len, 128, hidden=h_in, bm_shrink=bm_shrink, bm_expand=32,
+                        ksplit=ksplit, reduce_in_expand=rie)
+        y = y0.to(dev)
+        plan.apply(y, x.to(dev), pd.key_buffer, pd.value_buffer, pd.a_start, pd.a_len, pd.a_loc, 2, pd.a_scaling)
+        assert_parity(y.cpu(), want, f"ksplit {ksplit} h_in {h_in} bm {bm_shrink} rie {rie}")
+        assert torch.equal(y.cpu()[ids < 0], y0[ids < 0])
