@@ -129,3 +129,39 @@ def test_delora_compensation(dev, n):
     has = w.ids >= 0
     err = (out - ref)[has].abs().max()
     assert err <= (6e-2 if w.dtype == torch.bfloat16 else 8e-3) * (1 + ref[has].abs().max()), err
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_merge_random_shapes(dev, seed):
+    """Non-square weights, widths that are multiples of 8 only, 1-5 pool slots, any subset of slots,
+    weights that are column slices of a wider matrix (whose other columns must stay untouched)."""
+    import random
+    rnd = random.Random(seed)
+    dtype = rnd.choice([torch.float16, torch.bfloat16])
+    h_in, h_out = (rnd.choice([8, 24, 72, 136, 264, 520, 1000, 1032, 2056]) for _ in range(2))
+    ranks = [rnd.choice([8, 16, 24, 32, 40, 64, 128]) for _ in range(rnd.choice([1, 2, 4]))]
+    n_slots = rnd.choice([1, 2, 4, 5])
+    slots = rnd.sample(range(n_slots), rnd.randint(1, min(4, n_slots)))
+    adapter, scaling, sign = rnd.randrange(len(ranks)), rnd.choice([1.0, 2.0, 0.5, 1.7, 0.3]), rnd.choice([1, -1])
+    pad = rnd.choice([0, 8, 64])
+    what = f"seed {seed} {dtype} {h_in}x{h_out} ranks {ranks} slots {slots}/{n_slots} s {scaling} sign {sign} pad {pad}"
+    print(what, flush=True)
+    g = torch.Generator().manual_seed(seed)
+    pool = W.make_pool(ranks, h_in, h_out, dtype, g, True, n_slots=n_slots, std=0.05, heads=1)
+    Ws = [(torch.randn(h_in, h_out, generator=g) * 0.05).to(dtype) for _ in slots]
+    want = O.merge_adapter(Ws, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, adapter,
+                           scaling, slots=slots, n_slots=n_slots, sign=sign)
+    big = [torch.zeros(h_in, h_out + pad, dtype=dtype, device=dev) for _ in Ws]
+    for b, w in zip(big, Ws):
+        b[:, :h_out] = w.to(dev)
+    Wd = [b[:, :h_out] for b in big]
+    p = pool.to(dev)
+    fn = merge_adapter if sign > 0 else unmerge_adapter
+    fn(Wd, p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, adapter, scaling, max(ranks), slots=slots,
+       n_slots=n_slots)
+    for k in range(len(slots)):
+        d = (Wd[k].cpu().float() - want[k].float()).abs()
+        lim = 2 * ulp_of(torch.maximum(want[k].float().abs(), Ws[k].float().abs()).to(dtype))
+        assert (d <= lim).all(), what + f" target {k}: more than one ulp of ab"
+        assert (d > 0).float().mean() < 0.03, what
+        assert not big[k][:, h_out:].any(), what + " wrote outside the weight's columns"
