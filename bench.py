@@ -236,6 +236,7 @@ def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0, only_tar
     if not only:
         report["adapter_residency"] = bench_adapter_residency(torch, dev)
         report["config5_step"] = bench_config5_step(torch, W, dev, use_graph)
+        report["config4_prefill_step"] = bench_config4_prefill_step(torch, W, dev, use_graph)
     with open(path, "w") as f:
         json.dump(report, f, indent=1)
 
@@ -309,6 +310,47 @@ def bench_config5_step(torch, W, dev, use_graph):
     out["tokens"] = T
     out["lora_calls_per_layer"] = 4
     return out
+
+
+def bench_config4_prefill_step(torch, W, dev, use_graph, n_layers=8):
+    """LoRA inside a prefill forward pass of benchmark configuration 4 (16 requests of 256 image + 16..128 text
+    tokens, 16 adapters of rank 64, LoRA on all 7 projections): `n_layers` decoder layers of the 7B shape with
+    stock PyTorch `mm` and per-request causal attention around the LoRA calls.  Reported per layer: base only,
+    with LoRA, and the difference -- what the ops cost when y has just been written by the base projection and
+    is read again right after, as opposed to the back-to-back figures of the per-target report."""
+    from valora_amd.layer import LayerPlans, LayerPools, LayerWeights, layer_forward, segment_attention
+    H, MLP, heads, dt = 4096, 11008, 32, torch.bfloat16
+    w4 = W.CONFIGS[4]()
+    wd = w4.to(dev)
+    pa, pu, pdn = wd.target("q").pool, wd.target("gate").pool, wd.target("down").pool
+    idx = (pa.a_start, pa.a_len, pa.a_loc, pa.a_scaling)
+    g = torch.Generator(device=dev).manual_seed(44)
+    rnd = lambda *shape, s=1.0: (torch.randn(*shape, device=dev, generator=g) * s).to(dt)
+    layers = []
+    for _ in range(n_layers):
+        wts = LayerWeights(rnd(H, H, s=H ** -0.5), rnd(H, H, s=H ** -0.5), rnd(H, H, s=H ** -0.5), rnd(H, H, s=H ** -0.5),
+                           rnd(H, MLP, s=H ** -0.5), rnd(H, MLP, s=H ** -0.5), rnd(MLP, H, s=MLP ** -0.5),
+                           torch.ones(H, device=dev, dtype=dt), torch.ones(H, device=dev, dtype=dt))
+        pools = LayerPools(tuple(rnd(*b.shape, s=0.02) for b in (pa.key_buffer, pa.value_buffer)),
+                           tuple(rnd(*b.shape, s=0.02) for b in (pu.key_buffer, pu.value_buffer)),
+                           tuple(rnd(*b.shape, s=0.02) for b in (pdn.key_buffer, pdn.value_buffer)), *idx)
+        layers.append((wts, pools))
+    plans = LayerPlans(wd.ids, pa.a_start, pa.a_len, max(pa.ranks), H, MLP)
+    attention = segment_attention([int(n) for n in w4.b_seq_len.tolist()], heads)
+    x0 = rnd(w4.T, H)
+
+    def step(lora):
+        x = x0
+        for wts, pools in layers:
+            x = layer_forward(x, wts, pools if lora else None, plans if lora else None, attention, heads)
+        return x
+
+    us = {}
+    for name, lora in (("base_only", False), ("with_lora", True)):
+        us[name] = min(time_graph(torch, lambda: step(lora), 5, 2, use_graph)[0] for _ in range(2)) * 1e3 / n_layers
+    return {"tokens": w4.T, "layers": n_layers, "us_per_layer_base_only": round(us["base_only"], 1),
+            "us_per_layer_with_lora": round(us["with_lora"], 1),
+            "lora_us_per_layer": round(us["with_lora"] - us["base_only"], 1), "lora_calls_per_layer": 4}
 
 
 def bench_adapter_residency(torch, dev):
