@@ -7,7 +7,7 @@ import torch
 
 from oracle import lora_oracle as O
 from valora_amd import workloads as W
-from tests._util import MAX_ABS, REL_L2, assert_parity, max_rank
+from tests._util import assert_parity
 
 pytestmark = pytest.mark.gpu
 

@@ -22,7 +22,7 @@ reference issues 8 calls (16 launches, each followed by a synchronize) for its f
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Callable, Dict, Optional, Tuple
+from typing import Callable, Optional, Tuple
 
 import torch
 import torch.nn.functional as F

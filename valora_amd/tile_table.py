@@ -16,7 +16,7 @@ import json
 import math
 import os
 from dataclasses import dataclass
-from typing import Dict, Tuple
+from typing import Dict
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 TABLE_PATH = os.path.join(_HERE, "tile_table.json")

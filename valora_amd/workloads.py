@@ -12,7 +12,7 @@ contiguous (valora/server/router/model_infer/infer_batch.py:60-110), per-token a
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, List, Optional, Tuple
+from typing import Dict, List, Tuple
 
 import torch
 
