@@ -22,11 +22,16 @@ Pinning status of each function (what fixes it besides its own text):
   operands (they must agree to rounding) and against fp64.
 * ``count_consecutive_requests`` -- pinned by brute force against ``itertools.groupby``.
 * ``set_sgmm_args`` -- pinned by hand-derived vectors held in ``tests/golden/segments.json``.
-* ``sgmm_*_literal`` (ATMM's literal run-time behaviour under its own quirks) -- follows the
-  source text only; no runnable reference artefact exercises it: PARITY UNPINNED beyond
-  the textbook grouped-GEMM closed form it reduces to.
+* ``sgmm_canonical`` -- ``bgmv_*`` applied to the rows the first P segments cover; pinned by a
+  plain-loop covered-rows mask and by ``P = number of runs`` reducing to ``bgmv_*``.  (ATMM's
+  literal launch -- adapter from an all-zero tensor, rank from an all-64 tensor, B read as
+  ``[r, H_out]``, scaling ignored -- is not restated: nothing is compared against it.)
 * ``triton_shrink`` / ``triton_expand`` -- same closed form as ``bgmv_*`` per request;
-  pinned by equivalence with ``bgmv_*`` through ``repeat_interleave``.
+  pinned by equivalence with ``bgmv_*`` through ``repeat_interleave`` and, for what differs from
+  BGMV (zero-filled columns up to the last column block, rows past the grid's last row block
+  left alone, accumulation into a non-zero ``o``), by a brute force that walks the Triton launch
+  grid program by program with the kernels' own masks and flat offsets on exact-arithmetic
+  (small-integer) operands.
 * ``merge_weight`` / ``merge_adapter`` -- a library GEMM plus an in-place add in the reference; pinned by
   small-integer cases where every product and sum is exact (bit-exact against plain Python loops
   over the pool indices), by fp64, by ``unmerge(merge(W))`` staying within one rounding of W, and by
@@ -125,11 +130,13 @@ def bgmv_shrink(y, x, w, a_start, a_len, a_loc, ids, slot, n_slots=N_SLOTS, acc=
 
 
 def bgmv_expand(y, x, w, a_start, a_len, a_loc, ids, slot, scales, n_slots=N_SLOTS,
-                acc=torch.float32):
+                acc=torch.float32, round_y=True):
     """``y[t,o] = T( f32(y[t,o]) + sum_{j<r} f32(x[t,j]) * f32(B[j,o]) * f32(scale[a]) )``.
 
     valora/csrc/bgmv/bgmv_impl.cuh:152-207: lanes with ``j >= r`` contribute zero (:186-188),
     scale is read as T and widened (:180,197), the read-modify-write rounds once (:205-207).
+    ``round_y=False`` returns the accumulator before that last rounding (what the tolerance
+    accounting of the parity tests places between two neighbouring T values).
     """
     T = y.dtype
     h_out = y.shape[1]
@@ -147,7 +154,7 @@ def bgmv_expand(y, x, w, a_start, a_len, a_loc, ids, slot, scales, n_slots=N_SLO
         sel = torch.tensor([i for i, v in enumerate(ids_l) if v == a], dtype=torch.long)
         s = _f(scales, acc)[a]
         out[sel] += (xv[sel, :r] @ B) * s
-    return round_to(out, T)
+    return round_to(out, T) if round_y else out
 
 
 def dispatch_bgmv(y, x, w, a_start, a_len, a_loc, ids, qkvo, scales):
@@ -172,7 +179,7 @@ def dispatch_bgmv(y, x, w, a_start, a_len, a_loc, ids, qkvo, scales):
 
 
 def lora_op(y, x, kb, vb, a_start, a_len, a_loc, ids, slot, scales, n_slots=N_SLOTS,
-            acc=torch.float32, round_v=True):
+            acc=torch.float32, round_v=True, round_y=True):
     """Shrink then expand with the intermediate held exactly as the reference holds it.
 
     The reference stores ``delta`` as a T tensor between the two launches
@@ -185,7 +192,7 @@ def lora_op(y, x, kb, vb, a_start, a_len, a_loc, ids, slot, scales, n_slots=N_SL
     if round_v:
         v = torch.zeros(x.shape[0], R, dtype=T)
         v = bgmv_shrink(v, x, kb, a_start, a_len, a_loc, ids, slot, n_slots, acc)
-        return bgmv_expand(y, v, vb, a_start, a_len, a_loc, ids, slot, scales, n_slots, acc)
+        return bgmv_expand(y, v, vb, a_start, a_len, a_loc, ids, slot, scales, n_slots, acc, round_y)
     out = _f(y, acc).clone()
     ids_l = ids.tolist()
     for a in sorted(set(ids_l)):
@@ -307,36 +314,6 @@ def sgmm_canonical(y, x, w, a_start, a_len, a_loc, ids, qkvo, scales, output_cou
     if x.shape[1] < y.shape[1]:
         return bgmv_expand(y, x, w, a_start, a_len, a_loc, eff, qkvo, scales)
     return bgmv_shrink(y, x, w, a_start, a_len, a_loc, eff, qkvo)
-
-
-def sgmm_literal(y, x, w, a_start, a_len, a_loc, qkvo, output_counts, rank_counts, lora_ids,
-                 start_ids, num_problems):
-    """What the ATMM launch literally computes (PARITY UNPINNED: source reading only).
-
-    For problem i: ``m = output_counts[i]``; adapter ``lora_ids[i]``; rank ``rank_counts[i]``;
-    weight base = ``w + a_loc[a_start[id] + rank*qkvo] * H`` read as **physically contiguous**
-    rows (atmm/valora/csrc/bgmv/bgmv_impl.cuh:85-97,110-123); shrink: ``Y_i += X_i * W_i`` with
-    W column-major ld=H_in (:157,96); expand: ``Y_i += X_i * W_i`` with W **row-major**
-    ``[rank, H_out]`` (:219,122); alpha = beta = 1, scaling ignored (:174,236).
-    """
-    T = y.dtype
-    out = _f(y).clone()
-    xf = _f(x)
-    h_in, h_out = x.shape[1], y.shape[1]
-    expand = h_in < h_out
-    wide = h_out if expand else h_in
-    wflat = _f(w).reshape(-1)
-    for i in range(int(num_problems)):
-        m, rk, a, s = int(output_counts[i]), int(rank_counts[i]), int(lora_ids[i]), int(start_ids[i])
-        row0 = int(a_loc[int(a_start[a]) + rk * qkvo])
-        blk = wflat[row0 * wide: row0 * wide + rk * wide]
-        if expand:
-            W = blk.reshape(rk, h_out)                    # [k, n] row-major
-            out[s: s + m] += xf[s: s + m, :rk] @ W
-        else:
-            W = blk.reshape(rk, h_in).T                   # column-major [k, n], ld = H_in
-            out[s: s + m, :rk] += xf[s: s + m] @ W
-    return round_to(out, T)
 
 
 def count_consecutive_requests(lora_rank: torch.Tensor, indicies: torch.Tensor):

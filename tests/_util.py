@@ -8,11 +8,11 @@ MAX_ABS = 2e-2   # tolerance stated by the benchmark definition: max-abs error
 REL_L2 = 1e-3    # and relative L2 error, both against the reference semantics with fp32 accumulation
 
 
-def oracle_target(w, name, round_v=True):
+def oracle_target(w, name, round_v=True, round_y=True):
     t = w.target(name)
     p = t.pool
     return O.lora_op(w.y0[name], w.x[t.h_in], p_kb(w, name), p.value_buffer, p.a_start, p.a_len, p.a_loc,
-                     w.ids, t.slot, p.a_scaling, round_v=round_v)
+                     w.ids, t.slot, p.a_scaling, round_v=round_v, round_y=round_y)
 
 
 def p_kb(w, name):
@@ -102,17 +102,35 @@ def ulp(want):
     return torch.pow(2.0, torch.floor(torch.log2(mag)) - bits)
 
 
-def assert_parity(got, want, what=""):
-    """max-abs <= 2e-2 and rel-L2 <= 1e-3.  Both sides are 16-bit tensors: where one unit in the
-    last place of the format is itself larger than 2e-2 (bf16 from |y| >= 4, fp16 from |y| >= 32)
-    a difference of that single ulp -- two roundings of fp32 sums that differ in the last bits --
-    is accepted, nothing larger."""
+# what -> (elements over the strict 2e-2, elements compared); filled by assert_parity
+ALLOWANCE = {}
+
+
+def assert_parity(got, want, what="", unrounded=None):
+    """max-abs <= 2e-2 and rel-L2 <= 1e-3.  Both sides are 16-bit tensors, so where one unit in the last
+    place of the format is itself larger than 2e-2 (bf16 from |y| >= 4, fp16 from |y| >= 32) two correct
+    fp32 accumulations that differ in their last bits can round to neighbouring values.  An element over
+    the strict 2e-2 is accepted only if it is such a pair: ``got`` and ``want`` are adjacent values of the
+    format (bit patterns differ by one) and, when ``unrounded`` (the oracle's accumulator before its
+    last rounding) is given, that value lies between the two.  The number of elements that used the
+    allowance is recorded in ``ALLOWANCE[what]``."""
     got, want = got.detach().cpu(), want.detach().cpu()
     err = (got.double() - want.double()).abs()
-    lim = torch.full_like(err, MAX_ABS)
-    if want.dtype in (torch.float16, torch.bfloat16):
-        lim = torch.maximum(lim, ulp(want))
     ma, rl = float(err.max()) if err.numel() else 0.0, O.rel_l2(got, want)
-    bad = int((err > lim).sum())
-    assert bad == 0 and rl <= REL_L2, f"{what}: max_abs={ma:.3e} rel_l2={rl:.3e} over_limit={bad}"
+    over = err > MAX_ABS
+    n_over = int(over.sum())
+    ALLOWANCE[what] = (n_over, got.numel())
+    assert rl <= REL_L2, f"{what}: max_abs={ma:.3e} rel_l2={rl:.3e}"
+    if n_over:
+        assert want.dtype in (torch.float16, torch.bfloat16) and got.dtype == want.dtype, \
+            f"{what}: max_abs={ma:.3e} over {MAX_ABS} on {n_over} elements"
+        g, w = got[over], want[over]
+        step = (g.view(torch.int16).int() - w.view(torch.int16).int()).abs()
+        bad = int((step != 1).sum())
+        assert bad == 0, f"{what}: max_abs={ma:.3e}; {bad} of {n_over} elements over {MAX_ABS} are more than one ulp apart"
+        if unrounded is not None:
+            u = unrounded.detach().cpu().double()[over]
+            lo, hi = torch.minimum(g.double(), w.double()), torch.maximum(g.double(), w.double())
+            outside = int(((u < lo) | (u > hi)).sum())
+            assert outside == 0, f"{what}: {outside} of {n_over} one-ulp differences do not straddle the unrounded value"
     return ma, rl

@@ -237,6 +237,159 @@ def test_triton_style_equals_bgmv_through_repeat_interleave():
     assert torch.equal(tri, be)
 
 
+# ------------------------------------------------------------------ Triton launch grid, program by program
+def _cdiv(a, b):
+    return -(-a // b)
+
+
+def _int_case(seed, seq, req, ranks, hidden, o_cols, dtype=torch.float16):
+    """Small-integer operands: every product and every partial sum is exactly representable in fp16 /
+    bf16 / fp32, so any summation order gives the same bits and the comparison can be exact."""
+    g = torch.Generator().manual_seed(seed)
+    pool = W.make_pool(list(ranks), hidden, hidden, dtype, g, True, std=1.0)
+    n = pool.n_rows
+    kb = torch.randint(-1, 2, (n, hidden), generator=g).to(dtype)
+    vb = torch.randint(-1, 2, (n, hidden), generator=g).to(dtype)
+    seq = torch.tensor(seq, dtype=torch.int32)
+    start = (torch.cumsum(seq, 0) - seq).to(torch.int32)
+    T = int(seq.sum())
+    x = torch.randint(-2, 3, (T, hidden), generator=g).to(dtype)
+    v = torch.randint(-2, 3, (T, o_cols), generator=g).to(dtype)
+    o0 = torch.randint(-3, 4, (T, o_cols), generator=g).to(dtype)
+    y0 = torch.randint(-3, 4, (T, hidden), generator=g).to(dtype)
+    scale = torch.tensor([0.5, 1.0, 2.0, 1.5][:len(ranks)], dtype=dtype)
+    return pool, kb, vb, seq, start, torch.tensor(req), x, v, o0, y0, scale
+
+
+def _grid_shrink(X, Wt, Out, b_loc, b_lora_start, b_lora_ranks, b_start_loc, b_seq_len, b_indicies, hidden,
+                 qkvo, max_rank, max_input_len):
+    """_shrink_fwd_kernel + its launcher (lora_prefill.py:56-102,139-163) on flat arrays: one loop
+    iteration per Triton program, masks and offsets as written there."""
+    BLOCK_N = 16 if max_rank > 8 else max_rank
+    BLOCK_M = 32
+    sx, sw, so = X.shape[1], Wt.shape[1], Out.shape[1]
+    Xf, Wf, Of = X.reshape(-1).tolist(), Wt.reshape(-1).tolist(), Out.reshape(-1).clone()
+    for cur_batch in range(len(b_seq_len)):
+        for start_n in range(_cdiv(max_rank, BLOCK_N)):
+            for start_m in range(_cdiv(max_input_len, BLOCK_M)):
+                ad = int(b_indicies[cur_batch])
+                seq_len = int(b_seq_len[cur_batch])
+                rank = int(b_lora_ranks[ad]) // 4
+                a0 = int(b_lora_start[ad]) + rank * qkvo
+                t0 = int(b_start_loc[cur_batch])
+                for mi in range(BLOCK_M):
+                    m = start_m * BLOCK_M + mi
+                    if not m < seq_len:        # store mask (:100); masked x rows load 0.0 and are never stored
+                        continue
+                    for ni in range(BLOCK_N):
+                        nn = start_n * BLOCK_N + ni
+                        acc = 0.0
+                        if nn < rank:          # weight mask (:89,96): other = 0.0
+                            w_loc = int(b_loc[a0 + nn])
+                            for k in range(hidden):
+                                acc += Xf[(t0 + m) * sx + k] * Wf[w_loc * sw + k]
+                        Of[(t0 + m) * so + nn] = acc
+    return Of.reshape(Out.shape)
+
+
+def _grid_expand(X, Wt, Out, scale, b_loc, b_lora_start, b_lora_ranks, b_start_loc, b_seq_len, b_indicies,
+                 feat_out, qkvo, max_rank, max_input_len):
+    """_expand_fwd_kernel + its launcher (lora_prefill.py:9-54,105-135), program by program."""
+    BLOCK_N, BLOCK_M = 128, 32
+    TILE = BLOCK_N
+    sx, sw, so = X.shape[1], Wt.shape[1], Out.shape[1]
+    Xf, Wf = X.reshape(-1).tolist(), Wt.reshape(-1).tolist()
+    Of = Out.reshape(-1).double().clone()
+    for cur_batch in range(len(b_seq_len)):
+        for cur_tile in range(_cdiv(feat_out, TILE)):
+            for start_m in range(_cdiv(max_input_len, BLOCK_M)):
+                ad = int(b_indicies[cur_batch])
+                seq_len = int(b_seq_len[cur_batch])
+                rank = int(b_lora_ranks[ad]) // 4
+                a0 = int(b_lora_start[ad]) + rank * qkvo
+                t0 = int(b_start_loc[cur_batch])
+                sc = float(scale[ad])
+                for start_n in range(cur_tile * TILE, (cur_tile + 1) * TILE, BLOCK_N):
+                    for ni in range(BLOCK_N):
+                        nn = start_n + ni
+                        assert nn < feat_out, "the emulation covers widths that are multiples of 128"
+                        w_loc = int(b_loc[a0 + (nn * rank) // feat_out])
+                        for mi in range(BLOCK_M):
+                            m = start_m * BLOCK_M + mi
+                            if not m < seq_len:
+                                continue
+                            acc = 0.0
+                            for d in range(max_rank):
+                                if d < rank:   # weight mask (:43); x is read for every d < BLOCK_RANK
+                                    acc += Xf[(t0 + m) * sx + d] * Wf[w_loc * sw + (nn * rank + d) % feat_out]
+                            Of[(t0 + m) * so + nn] += acc * sc
+    return Of.reshape(Out.shape)
+
+
+@pytest.mark.parametrize("max_rank,o_cols", [(8, 8), (8, 16), (24, 32), (16, 16), (32, 40)])
+def test_triton_shrink_vs_launch_grid(max_rank, o_cols):
+    """Non-zero o, ranks below max_rank (zero fill up to the last column block), a column block that
+    ends past max_rank (24 -> 32 columns), max_input_len shorter than the longest request (rows past
+    the last 32-row block keep their value), an empty request."""
+    ranks = [r for r in (8, 16, 24, 32) if r <= max_rank] or [8]
+    seq = [37, 1, 0, 70, 33]
+    req = [(i * 3) % len(ranks) for i in range(len(seq))]
+    H = 32
+    pool, kb, vb, seq, start, req, x, v, o0, y0, scale = _int_case(100 + max_rank, seq, req, ranks, H, o_cols)
+    for mx in (int(seq.max()), 40, 1):
+        want = _grid_shrink(x.double(), kb.double(), o0.double(), pool.a_loc, pool.a_start, pool.a_len, start,
+                            seq, req, H, 1, max_rank, mx)
+        got = O.triton_shrink(x, kb, o0, pool.a_loc, pool.a_start, pool.a_len, start, seq, req, H, 1, max_rank, mx)
+        assert torch.equal(got.double(), want), f"max_input_len={mx}"
+        # the case means something: some rows were left alone, some columns were zero-filled
+        if mx == 40:
+            assert torch.equal(got[int(start[3]) + 64:int(start[3]) + 70], o0[int(start[3]) + 64:int(start[3]) + 70])
+            assert not torch.equal(got[int(start[3]):int(start[3]) + 64], o0[int(start[3]):int(start[3]) + 64])
+
+
+@pytest.mark.parametrize("max_rank", [8, 16, 24])
+def test_triton_expand_vs_launch_grid(max_rank):
+    ranks = [r for r in (8, 16, 24) if r <= max_rank]
+    seq = [37, 1, 0, 70, 33]
+    req = [(i * 2) % len(ranks) for i in range(len(seq))]
+    H = 384     # every rank divides it, so an output's r weights never straddle two pool rows
+    pool, kb, vb, seq, start, req, x, v, o0, y0, scale = _int_case(200 + max_rank, seq, req, ranks, H, max_rank)
+    for mx in (int(seq.max()), 40):
+        want = _grid_expand(v.double(), vb.double(), y0, scale, pool.a_loc, pool.a_start, pool.a_len, start, seq,
+                            req, H, 2, max_rank, mx)
+        got = O.triton_expand(v, vb, y0, scale, pool.a_loc, pool.a_start, pool.a_len, start, seq, req, H, 2,
+                              max_rank, mx)
+        assert torch.equal(got.double(), want), f"max_input_len={mx}"
+        if mx == 40:
+            assert torch.equal(got[int(start[3]) + 64:int(start[3]) + 70], y0[int(start[3]) + 64:int(start[3]) + 70])
+
+
+def test_sgmm_canonical_covered_rows():
+    """Rows of the first P segments get the BGMV result, every other row keeps its bits; with P = all
+    runs the function is dispatch_bgmv (plain-loop mask, segment tensors with tails of ones)."""
+    pool, ids, x, y0, v, scales, R = _rand_case(21, T=40, H=64, ranks=(8, 16, 8))
+    ids = torch.repeat_interleave(torch.tensor([2, 0, 0, 1, 2]), torch.tensor([7, 9, 4, 12, 8]))
+    oc, rc, li, st = O.count_consecutive_requests(pool.a_len, ids)
+    assert oc == [7, 13, 12, 8]
+    oc_t = torch.tensor(oc + [1] * 3); st_t = torch.tensor(st + [1] * 3)
+    full_s = O.bgmv_shrink(torch.full((40, R), 1.5, dtype=x.dtype), x, pool.key_buffer, pool.a_start, pool.a_len,
+                           pool.a_loc, ids, 1)
+    full_e = O.bgmv_expand(y0, v, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, 1, scales)
+    for P in range(0, 5):
+        covered = [False] * 40
+        for i in range(P):
+            for t in range(st[i], st[i] + oc[i]):
+                covered[t] = True
+        cov = torch.tensor(covered)
+        d0 = torch.full((40, R), 1.5, dtype=x.dtype)
+        got = O.sgmm_canonical(d0, x, pool.key_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, 1, scales, oc_t,
+                               st_t, P)
+        assert torch.equal(got[cov], full_s[cov]) and torch.equal(got[~cov], d0[~cov])
+        got = O.sgmm_canonical(y0, v, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, 1, scales, oc_t,
+                               st_t, P)
+        assert torch.equal(got[cov], full_e[cov]) and torch.equal(got[~cov], y0[~cov])
+
+
 # ------------------------------------------------------------------ integer builders
 def test_count_consecutive_vs_groupby():
     g = torch.Generator().manual_seed(1)
