@@ -185,6 +185,21 @@ int mlora_dispatch_bgmv(void *stream, void *y, const void *x, const mlora_pool *
                         int64_t h_in, int64_t h_out, mlora_dtype dtype, void *workspace,
                         size_t workspace_bytes);
 
+/* mlora_dispatch_bgmv for callers that cannot allocate device memory and have no workspace to
+ * bring: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference.  Same arguments, checks, kernels and results as
+ * mlora_dispatch_bgmv, but the plan and the split-K partials live in a workspace of
+ * MLORA_STATIC_WORKSPACE_BYTES that is part of the library's device image (one copy per GPU, held
+ * until the process ends).  A call whose mlora_workspace_bytes(T, n_adapters, min(h_in, h_out))
+ * exceeds that size fails with MLORA_ERR_WORKSPACE and touches nothing.  The call allocates and
+ * frees nothing; the first call on each device looks the workspace's address up once (make that
+ * call outside a graph capture).  All calls on one GPU share the workspace: calls that overlap in
+ * time on one GPU (two streams, two threads) race, whereas calls queued on one stream are safe.   */
+#define MLORA_STATIC_WORKSPACE_BYTES (16u << 20)
+int mlora_dispatch_bgmv_static(void *stream, void *y, const void *x, const mlora_pool *pool,
+                               const int64_t *indicies, int64_t qkvo, const void *lora_scales,
+                               int64_t T, int64_t h_in, int64_t h_out, mlora_dtype dtype);
+
 /* dispatch_bgmv of the ATMM extension (imported as dispatch_sgmm)
  * atmm/valora/csrc/lora_ops.cc:115-186.  Rows of problems i < num_problems are processed with
  * the adapter named by their per-token id; tile arguments tb_* / wp_* are accepted and ignored

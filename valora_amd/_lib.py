@@ -24,7 +24,7 @@ SYMBOLS = [
     "mlora_last_error", "mlora_version", "mlora_plan_bytes", "mlora_scratch_bytes",
     "mlora_workspace_bytes", "mlora_build_plan", "mlora_count_consecutive",
     "mlora_ids_from_segments", "mlora_ids_from_requests", "mlora_shrink", "mlora_expand", "mlora_lora_apply",
-    "mlora_lora_apply_multi", "mlora_lora_fused", "mlora_dispatch_bgmv",
+    "mlora_lora_apply_multi", "mlora_lora_fused", "mlora_dispatch_bgmv", "mlora_dispatch_bgmv_static",
     "mlora_dispatch_sgmm", "mlora_prefill_shrink", "mlora_prefill_expand",
     "mlora_pool_alloc", "mlora_pool_alloc_contiguous", "mlora_pool_free", "mlora_pool_fill",
     "mlora_pool_scatter_rows", "mlora_pool_gather_rows", "mlora_index_compact", "mlora_merge_adapter",
@@ -90,6 +90,8 @@ def lib():
                                    POINTER(Pool), POINTER(Pool), c_int32, c_void_p, c_int32, c_int]
     L.mlora_dispatch_bgmv.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,
                                       c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t]
+    L.mlora_dispatch_bgmv_static.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,
+                                             c_void_p, c_int64, c_int64, c_int64, c_int]
     L.mlora_dispatch_sgmm.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,
                                       c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                       c_int, c_int32, c_void_p, c_size_t]

@@ -1,6 +1,7 @@
 // C ABI of libmlora: argument validation, workspace carving and kernel dispatch.
 // The checks mirror the reference's host-side checks (valora/csrc/lora_ops.cc:79-98,124-125);
 // failures come back as a status code plus a thread-local message instead of a C++ exception.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -550,6 +551,58 @@ int mlora_dispatch_sgmm(void *stream, void *y, const void *x, const mlora_pool *
   if (int rc = mlora_ids_from_segments(stream, ids_eff, indicies, start_ids, output_counts, num_problems, T)) return rc;
   return one_call(stream, y, x, pool, ids_eff, qkvo, lora_scales, T, h_in, h_out, dtype, shrink_mode, 0, 0, ws,
                   "dispatch_sgmm");
+}
+
+// ---- dispatch_bgmv for callers that cannot allocate --------------------------------------------
+// The workspace of mlora_dispatch_bgmv (plan + split-K partials) lives in this array instead of in
+// memory the caller brings.  Every device that loads the library holds its own copy until the
+// process ends.  Host code must never pass the array's name to a kernel (it is a host-side stand-in,
+// not a device address): the address is looked up once per device and kept in g_static_ws.
+constexpr size_t STATIC_WS_BYTES = (size_t)MLORA_STATIC_WORKSPACE_BYTES;
+constexpr int STATIC_WS_MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char scratch[STATIC_WS_BYTES];
+static std::atomic<void *> g_static_ws[STATIC_WS_MAX_DEVICES];
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+static int static_workspace(void **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(MLORA_ERR_LAUNCH, "dispatch_bgmv_static: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= STATIC_WS_MAX_DEVICES)
+    return fail(MLORA_ERR_INVALID, "dispatch_bgmv_static: device %d outside [0,%d)", dev, STATIC_WS_MAX_DEVICES);
+  void *p = g_static_ws[dev].load(std::memory_order_acquire);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(MLORA_ERR_LAUNCH, "dispatch_bgmv_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_static_ws[dev].store(p, std::memory_order_release);   // every thread gets the same address for a device
+  }
+  *out = p;
+  return MLORA_OK;
+}
+
+int mlora_dispatch_bgmv_static(void *stream, void *y, const void *x, const mlora_pool *pool, const int64_t *indicies,
+                               int64_t qkvo, const void *lora_scales, int64_t T, int64_t h_in, int64_t h_out,
+                               mlora_dtype dtype) {
+  if (int rc = check_dtype(dtype, h_in, h_out)) return rc;
+  if (int rc = check_pool(pool, "dispatch_bgmv_static")) return rc;
+  if (T < 0 || T > MAX_TOKENS) return fail(MLORA_ERR_INVALID, "dispatch_bgmv_static: T=%lld out of range", (long long)T);
+  if (T > 0 && (!y || !x || !indicies)) return fail(MLORA_ERR_INVALID, "dispatch_bgmv_static: null pointer");
+  if (T > 0 && h_in < h_out && !lora_scales) return fail(MLORA_ERR_INVALID, "dispatch_bgmv_static: lora_scales is null");
+  const int64_t narrow = h_in < h_out ? h_in : h_out;
+  const size_t need = mlora_workspace_bytes(T, pool->n_adapters, narrow);
+  if (need > STATIC_WS_BYTES)
+    return fail(MLORA_ERR_WORKSPACE,
+                "dispatch_bgmv_static: T=%lld with %lld adapters and rank %lld needs %zu bytes of workspace, the "
+                "built-in one has %zu; use mlora_dispatch_bgmv with a workspace of your own",
+                (long long)T, (long long)pool->n_adapters, (long long)narrow, need, STATIC_WS_BYTES);
+  void *ws_dev = nullptr;
+  if (int rc = static_workspace(&ws_dev)) return rc;
+  // nothing in the workspace has to start at zero: the plan kernel writes every word the later
+  // kernels read, and every split-K partial is written before it is summed
+  Carver ws{static_cast<char *>(ws_dev), STATIC_WS_BYTES};
+  return one_call(stream, y, x, pool, indicies, qkvo, lora_scales, T, h_in, h_out, dtype, MLORA_SHRINK_OVERWRITE, 0, 0,
+                  ws, "dispatch_bgmv_static");
 }
 
 int mlora_prefill_shrink(void *stream, void *o, const void *x, const mlora_pool *pool, const int32_t *b_start_loc,
