@@ -42,8 +42,8 @@ def parse():
     ap.add_argument("--bm-expand", type=int, default=None)
     ap.add_argument("--ksplit", type=int, default=None)
     ap.add_argument("--reduce-in-expand", type=int, default=None, help="1: expand sums the split-K chunks, 0: shrink does")
-    ap.add_argument("--fused", action="store_true", help="use the single-launch fused kernel instead of shrink + expand")
-    ap.add_argument("--replicas", type=int, default=0, help="output slices per tile of the fused kernel (0 = default)")
+    ap.add_argument("--one-launch", type=int, default=None,
+                    help="1: shrink and expand as work items of one grid, 0: two launches (default: the tile table's choice)")
     ap.add_argument("--pmc-copy-mib", type=int, default=0,
                     help="first run one plain device copy of this many MiB: a kernel of known traffic to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings with")
@@ -451,22 +451,18 @@ def main():
     w, wd, kb, vb, xs, ys = build_layers(torch, W, dev, L)
     t = wd.targets[0]
     p = t.pool
-    if args.fused and args.bm_shrink is None:
-        args.bm_shrink = 16
     plan = LoraPlan(wd.ids, p.a_start, p.a_len, 16, hidden=4096, bm_shrink=args.bm_shrink,
                     bm_expand=args.bm_expand, ksplit=args.ksplit,
-                    reduce_in_expand=None if args.reduce_in_expand is None else bool(args.reduce_in_expand))
+                    reduce_in_expand=None if args.reduce_in_expand is None else bool(args.reduce_in_expand),
+                    one_launch=None if args.one_launch is None else bool(args.one_launch))
     idx = (p.a_start, p.a_len, p.a_loc)
     use_graph = not args.no_graph
 
-    fused = args.fused
+    fused = plan.one_launch
 
     def step():
         for l in range(L):
-            if fused:
-                plan.apply_fused(ys[l], xs[l], kb[l], vb[l], *idx, 0, p.a_scaling, args.replicas)
-            else:
-                plan.apply(ys[l], xs[l], kb[l], vb[l], *idx, 0, p.a_scaling)
+            plan.apply(ys[l], xs[l], kb[l], vb[l], *idx, 0, p.a_scaling)
 
     def shrink_only():
         for l in range(L):
@@ -514,7 +510,7 @@ def main():
     bytes_op = w.algorithmic_bytes("q")
     assert bytes_op == bytes_shrink + bytes_expand
     if fused:
-        dom = ("fused_kernel", bytes_op, op_us)
+        dom = ("decode_kernel", bytes_op, op_us)
     else:
         dom = ("expand_kernel", bytes_expand, ex_us) if ex_us >= sh_us else ("shrink_kernel", bytes_shrink, sh_us)
     achieved = dom[1] / (dom[2] * 1e-6) / 1e9
@@ -534,7 +530,7 @@ def main():
                                "4096->4096, fp16, shrink+expand; one step = this op on %d layers" % L,
                    "layers_per_step": L, "tokens": w.T, "adapters_touched": len(used),
                    "launch": "hip graph replay" if use_graph else "eager python launches",
-                   "kernels": "fused shrink+expand, one launch" if fused else "shrink then expand, two launches",
+                   "kernels": "shrink and expand items of one grid, one launch" if fused else "shrink then expand, two launches",
                    "tile": {"bm_shrink": plan.bm_shrink, "ksplit": plan.ksplit, "bm_expand": plan.bm_expand}},
         "hbm_gbps": round(bytes_op / (us_per_layer * 1e-6) / 1e9, 1),
         "hbm_frac": round(bytes_op / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),

@@ -39,10 +39,24 @@ enum {
 
 /* flags of mlora_shrink / mlora_expand / mlora_lora_apply */
 enum {
-  MLORA_REDUCE_IN_EXPAND = 1  /* split-K chunks are summed by the expand launch instead of by a
+  MLORA_REDUCE_IN_EXPAND = 1, /* split-K chunks are summed by the expand launch instead of by a
                                  separate reduce launch: one launch fewer for small batches, more
                                  re-reads for large ones.  Must be given to both launches of a pair,
                                  with the same ksplit.                                            */
+  MLORA_ONE_LAUNCH = 2,       /* mlora_lora_apply / mlora_lora_apply_multi only: shrink and expand are
+                                 work items of ONE grid; an expand item requests its B and y operands,
+                                 then waits (bounded) for its tile's K-chunk partials and computes them
+                                 itself if they do not come.  For decode-like batches: needs a plan cut
+                                 with bm_shrink = bm_expand = 16 and max_rank <= 64; ksplit is raised to
+                                 2 if smaller and cut so that ksplit * n_targets <= 16; scratch of
+                                 mlora_one_launch_scratch_bytes().  A batch whose grid the device cannot
+                                 hold all at once is run as two launches instead.  Bit-identical to the
+                                 two-launch op with
+                                 MLORA_REDUCE_IN_EXPAND and the same ksplit.  Launches that share a plan
+                                 must not overlap in time.                                        */
+  MLORA_ONE_LAUNCH_NO_WAIT = 4 /* with MLORA_ONE_LAUNCH: expand items do not wait at all and always
+                                 compute their tile's partials themselves (the give-up path made
+                                 testable; same results, slower)                                  */
 };
 
 /* Pool + adapter index operands shared by all op entry points (device pointers).
@@ -78,6 +92,10 @@ size_t mlora_plan_bytes(int64_t T, int64_t n_adapters);
 /* Bytes of the scratch buffer that carries v = x*A^T from mlora_shrink to mlora_expand (a T-typed
  * [T, max_rank] matrix plus, for ksplit > 1, the fp32 split-K partials).                       */
 size_t mlora_scratch_bytes(int64_t T, int64_t max_rank, int32_t ksplit);
+/* Bytes of scratch a call with MLORA_ONE_LAUNCH needs (its K-chunk partials are laid out tile by tile, in
+ * whole cache lines per tile, which takes more room than mlora_scratch_bytes gives).             */
+size_t mlora_one_launch_scratch_bytes(int64_t T, int64_t n_adapters, int64_t max_rank, int32_t ksplit,
+                                      int32_t n_targets);
 /* Bytes of scratch the one-call entry points (dispatch_bgmv, dispatch_sgmm, prefill_*) need.
  * Replaces sgmm_tmp_size (atmm/valora/csrc/bgmv/bgmv_impl.cuh:128-132).                       */
 size_t mlora_workspace_bytes(int64_t T, int64_t n_adapters, int64_t max_rank);
@@ -165,16 +183,6 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
                            const void *x, int64_t T, int64_t h_in, int64_t h_out, int64_t max_rank,
                            const mlora_pool *pool_a, int32_t n_targets, const mlora_target *targets,
                            const void *scales, int32_t ksplit, int32_t flags, mlora_dtype dtype);
-
-/* Shrink + expand of one target in ONE launch, for decode-like batches (few tokens per adapter):
- * each workgroup recomputes v for its tile of <= 16 tokens and expands one slice of the output
- * columns, so nothing is handed from one workgroup to another and no scratch is needed.
- * Requires a plan built with bm_shrink = 16 and max_rank <= 64.  replicas = number of output
- * slices per tile (0 = library default).  Same result as mlora_lora_apply.                    */
-int mlora_lora_fused(void *stream, const mlora_plan *plan, void *y, const void *x, int64_t T,
-                     int64_t h_in, int64_t h_out, int64_t max_rank, const mlora_pool *pool_a,
-                     const mlora_pool *pool_b, int32_t slot, const void *scales, int32_t replicas,
-                     mlora_dtype dtype);
 
 /* ---- the reference's entry points, one call each -------------------------------------------- */
 /* dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales)

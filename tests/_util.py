@@ -56,13 +56,15 @@ def run_multi(wd, names, **kw):
     return ys
 
 
-def run_fused(wd, name, replicas=0):
+def run_one_launch(wd, name, no_wait=False, ksplit=4):
+    """The one-launch op (shrink and expand items of one grid); ``no_wait``: every expand item takes its
+    give-up path and computes the tile's partials itself."""
     from valora_amd.plan import LoraPlan
     t = wd.target(name); p = t.pool
-    plan = LoraPlan(wd.ids, p.a_start, p.a_len, max_rank(wd), hidden=t.h_in, bm_shrink=16)
+    plan = LoraPlan(wd.ids, p.a_start, p.a_len, max_rank(wd), hidden=t.h_in, one_launch=True, ksplit=ksplit,
+                    one_launch_no_wait=no_wait)
     y = wd.y0[name].clone()
-    plan.apply_fused(y, wd.x[t.h_in], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot,
-                     p.a_scaling, replicas)
+    plan.apply(y, wd.x[t.h_in], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
     return y
 
 

@@ -9,7 +9,7 @@ import torch
 
 from oracle import lora_oracle as O
 from valora_amd import workloads as W
-from tests._util import (assert_parity, max_rank, oracle_target, run_bgmv, run_fused, run_multi, run_plan,
+from tests._util import (assert_parity, max_rank, oracle_target, run_bgmv, run_multi, run_one_launch, run_plan,
                          run_prefill, run_sgmm)
 
 pytestmark = pytest.mark.gpu
@@ -36,8 +36,12 @@ def test_small_configs_all_entry_points(dev, n):
         # and y -- bf16 carries 8 significant bits, so ~1e-3 relative is the floor for any implementation
         # that, like the reference, holds v as a 16-bit tensor
         assert O.rel_l2(got, exact) <= (4e-3 if w.dtype == torch.bfloat16 else 5e-4)
-        for rep in (0, 1, 3):
-            assert_parity(run_fused(wd, t.name, rep).cpu(), want, f"config{n}/{t.name}/fused rep={rep}")
+        if max_rank(w) <= 64:
+            for ks, no_wait in ((4, False), (2, True), (7, False)):
+                one = run_one_launch(wd, t.name, no_wait=no_wait, ksplit=ks)
+                assert_parity(one.cpu(), want, f"config{n}/{t.name}/one launch ks={ks} no_wait={no_wait}")
+                two = run_plan(wd, t.name, bm_shrink=16, bm_expand=16, ksplit=ks, reduce_in_expand=True)
+                assert torch.equal(one, two), f"config{n}/{t.name}: one launch differs from two launches (ks={ks})"
         if t.h_in == t.h_out:      # the reference's entry points decide the direction by h_in < h_out
             y, delta = run_bgmv(wd, t.name)
             assert_parity(y.cpu(), want, f"config{n}/{t.name}/bgmv")
@@ -93,8 +97,12 @@ def test_config2_full(dev, variant):
     want = oracle_target(w, "q")
     assert_parity(run_plan(wd, "q").cpu(), want, "config2/plan")
     assert_parity(run_bgmv(wd, "q")[0].cpu(), want, "config2/bgmv")
-    for rep in (0, 1, 2, 7, 64):
-        assert_parity(run_fused(wd, "q", rep).cpu(), want, f"config2/fused rep={rep}")
+    for ks in (2, 4, 8, 16):
+        two = run_plan(wd, "q", bm_shrink=16, bm_expand=16, ksplit=ks, reduce_in_expand=True)
+        for no_wait in (False, True):
+            one = run_one_launch(wd, "q", no_wait=no_wait, ksplit=ks)
+            assert_parity(one.cpu(), want, f"config2/one launch ks={ks} no_wait={no_wait}")
+            assert torch.equal(one, two), f"config2: one launch (no_wait={no_wait}) differs from two launches at ks={ks}"
     for ks in (1, 4, 16):
         for bm_s, bm_e in ((16, 16), (32, 64), (64, 256), (128, 128)):
             for rie in (False, True):
@@ -110,8 +118,8 @@ def test_full_configs_vs_oracle(dev, n, names):
     for name in names:
         want = oracle_target(w, name)
         assert_parity(run_plan(wd, name).cpu(), want, f"config{n}/{name}/plan")
-        if n == 5:  # the decode-heavy layer also goes through the single-launch kernel
-            assert_parity(run_fused(wd, name).cpu(), want, f"config{n}/{name}/fused")
+        if n == 5:  # the decode-heavy layer also goes through the one-launch op
+            assert_parity(run_one_launch(wd, name).cpu(), want, f"config{n}/{name}/one launch")
     sq = [t.name for t in w.targets if t.h_in == t.h_out][0]
     assert_parity(run_bgmv(wd, sq)[0].cpu(), oracle_target(w, sq), f"config{n}/{sq}/bgmv")
 
@@ -196,12 +204,11 @@ def test_full_size_properties(dev, n):
         # determinism
         assert torch.equal(base, run(wd.ids, x, y0, p.a_scaling))
         if n in (2, 5):
-            # the single-launch kernel is deterministic and token-permutation equivariant too
+            # the one-launch op is deterministic and token-permutation equivariant too
             def runf(ids, xx, yy):
-                plan = LoraPlan(ids, p.a_start, p.a_len, R, hidden=t.h_in, bm_shrink=16)
+                plan = LoraPlan(ids, p.a_start, p.a_len, R, hidden=t.h_in, one_launch=True)
                 out = yy.clone()
-                plan.apply_fused(out, xx, p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot,
-                                 p.a_scaling)
+                plan.apply(out, xx, p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
                 return out
             fb = runf(wd.ids, x, y0)
             assert torch.equal(fb, runf(wd.ids, x, y0))

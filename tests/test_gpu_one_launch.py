@@ -1,0 +1,210 @@
+"""GPU: the one-launch op (shrink and expand items of one grid, hand-off inside the launch).
+
+Its contract is "bit-identical to the two-launch op with the same ksplit whose expand sums the K chunks", on
+every path an item can take: partials handed over by the shrink items, partials recomputed because the wait
+was given up (forced from the host with a poll bound of zero -- no kernel is ever made to wait or hang), items
+the device cannot hold from the start, several targets in one call, and -- the part a single call cannot
+show -- launch after launch on one plan, where a stamp left behind by the previous launch must never be taken
+for a fresh one."""
+import random
+
+import pytest
+import torch
+
+from oracle import lora_oracle as O
+from valora_amd import workloads as W
+from valora_amd.plan import LoraPlan
+from tests._util import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(wd, name, R, hidden, ksplit, **kw):
+    t = wd.target(name); p = t.pool
+    one = LoraPlan(wd.ids, p.a_start, p.a_len, R, hidden=hidden, one_launch=True, ksplit=ksplit, **kw)
+    two = LoraPlan(wd.ids, p.a_start, p.a_len, R, hidden=hidden, one_launch=False, bm_shrink=16, bm_expand=16,
+                   ksplit=one.ksplit, reduce_in_expand=True)
+    assert one.one_launch and not two.one_launch
+    return one, two
+
+
+def test_launch_after_launch_on_one_plan(dev):
+    """32 'layers' with their own x, y and pool on ONE plan, three times over, single-target and three-target
+    calls interleaved (so the number of shrink items per tile changes from launch to launch): every result
+    equals the two-launch op's, bit for bit."""
+    w = W.config2(hidden=1024, n_tokens=200, n_adapters=48)
+    wd = w.to(dev)
+    t = wd.target("q"); p = t.pool
+    R = max(p.ranks)
+    one, two = _pair(wd, "q", R, 1024, 4)
+    g = torch.Generator(device=dev).manual_seed(5)
+    L = 32
+    kb = [(torch.randn(p.key_buffer.shape, generator=g, device=dev) * 0.05).to(w.dtype) for _ in range(4)]
+    vb = [(torch.randn(p.value_buffer.shape, generator=g, device=dev) * 0.05).to(w.dtype) for _ in range(4)]
+    xs = [torch.randn(w.T, 1024, generator=g, device=dev).to(w.dtype) for _ in range(L)]
+    y0 = [torch.randn(w.T, 1024, generator=g, device=dev).to(w.dtype) for _ in range(L)]
+    idx = (p.a_start, p.a_len, p.a_loc)
+    for rep in range(3):
+        got = [y.clone() for y in y0]
+        want = [y.clone() for y in y0]
+        for plan, ys in ((one, got), (two, want)):
+            for l in range(L):
+                if l % 5 == 3:     # a q+k+v style call: three targets share x
+                    trio = [ys[l], ys[(l + 1) % L], ys[(l + 2) % L]]
+                    plan.apply_multi(trio, xs[l], kb[l % 4], vb[l % 4], *idx, [0, 1, 2], p.a_scaling)
+                else:
+                    plan.apply(ys[l], xs[l], kb[l % 4], vb[l % 4], *idx, l % 4, p.a_scaling)
+        torch.cuda.synchronize()
+        for l in range(L):
+            assert torch.equal(got[l], want[l]), f"repetition {rep}, layer {l}"
+    # and the numbers are the operator's: one layer against the oracle
+    y = y0[0].clone()
+    one.apply(y, xs[0], kb[0], vb[0], *idx, 0, p.a_scaling)
+    ref = O.lora_op(y0[0].cpu(), xs[0].cpu(), kb[0].cpu(), vb[0].cpu(), p.a_start.cpu(), p.a_len.cpu(),
+                    p.a_loc.cpu(), w.ids, 0, p.a_scaling.cpu())
+    assert_parity(y.cpu(), ref, "one launch vs oracle")
+
+
+def test_graph_replays_of_a_layer_loop(dev):
+    """The benchmark's shape of use: a loop over layers on one plan captured in a HIP graph and replayed,
+    with eager work in between; every replay equals the eager two-launch result."""
+    w = W.config2(hidden=512, n_tokens=128, n_adapters=40)
+    wd = w.to(dev)
+    t = wd.target("q"); p = t.pool
+    one, two = _pair(wd, "q", max(p.ranks), 512, 4)
+    g = torch.Generator(device=dev).manual_seed(9)
+    L = 6
+    xs = [torch.randn(w.T, 512, generator=g, device=dev).to(w.dtype) for _ in range(L)]
+    y0 = [torch.randn(w.T, 512, generator=g, device=dev).to(w.dtype) for _ in range(L)]
+    ys = [y.clone() for y in y0]
+    idx = (p.a_start, p.a_len, p.a_loc)
+
+    def loop(plan, out):
+        for l in range(L):
+            plan.apply(out[l], xs[l], p.key_buffer, p.value_buffer, *idx, l % 4, p.a_scaling)
+
+    want = [y.clone() for y in y0]
+    loop(two, want)
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream(device=dev)
+    s.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(s):
+        loop(one, ys)                         # warm-up on the capture stream
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            loop(one, ys)
+    torch.cuda.current_stream(dev).wait_stream(s)
+    for i in range(5):
+        for y, src in zip(ys, y0):
+            y.copy_(src)
+        junk = torch.randn(1 << 20, device=dev).sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for l in range(L):
+            assert torch.equal(ys[l], want[l]), f"replay {i}, layer {l}"
+        assert torch.isfinite(junk)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_one_launch_random_shapes(dev, seed):
+    rnd = random.Random(500 + seed)
+    dtype = rnd.choice([torch.float16, torch.bfloat16])
+    T = rnd.choice([1, 2, 15, 16, 17, 33, 64, 100, 129, 256, 300])
+    h_in, h_out = rnd.choice([256, 264, 520, 1032, 2056, 4096]), rnd.choice([8, 72, 264, 520, 1000, 1032, 4096])
+    A = rnd.choice([1, 2, 5, 17, 64])
+    ranks = [rnd.choice([8, 16, 24, 32, 40, 64]) for _ in range(A)]
+    n_slots = rnd.choice([1, 2, 4, 5])
+    ks = rnd.choice([2, 3, 4, 5, 8, 16])
+    n_targets = rnd.choice([1, 1, 2, 3, 4])
+    no_wait = rnd.random() < 0.3
+    style = rnd.choice(["random", "sorted", "holes", "one"])
+    what = (f"seed {seed}: {dtype} T={T} {h_in}->{h_out} ranks={ranks[:6]}.. slots={n_slots} ks={ks} "
+            f"targets={n_targets} no_wait={no_wait} {style}")
+    print(what, flush=True)
+    g = torch.Generator().manual_seed(2000 + seed)
+    pool = W.make_pool(ranks, h_in, h_out, dtype, g, True, n_slots=n_slots, std=0.05,
+                       scalings=[0.25 + 0.5 * ((7 * i) % 5) for i in range(A)], heads=1, extra_rows=3)
+    if style == "random":
+        ids = torch.randint(0, A, (T,), generator=g)
+    elif style == "sorted":
+        ids = torch.randint(0, A, (T,), generator=g).sort().values
+    elif style == "holes":
+        ids = torch.randint(-1, A, (T,), generator=g)
+    else:
+        ids = torch.full((T,), A - 1, dtype=torch.long)
+    x = torch.randn(T, h_in, generator=g).to(dtype)
+    y0 = [torch.randn(T, h_out, generator=g).to(dtype) for _ in range(n_targets)]
+    slots = [(seed + i) % n_slots for i in range(n_targets)]
+    pd = pool.to(dev)
+    idx = (pd.a_start, pd.a_len, pd.a_loc)
+    R = max(ranks)
+    one = LoraPlan(ids.to(dev), pd.a_start, pd.a_len, R, n_slots=n_slots, hidden=h_in, one_launch=True, ksplit=ks,
+                   one_launch_no_wait=no_wait)
+    two = LoraPlan(ids.to(dev), pd.a_start, pd.a_len, R, n_slots=n_slots, hidden=h_in, one_launch=False,
+                   bm_shrink=16, bm_expand=16, ksplit=one.ksplit, reduce_in_expand=True)
+    xd = x.to(dev)
+    for rep in range(2):                       # twice on the same plan
+        got = [y.to(dev) for y in y0]
+        if n_targets == 1:
+            one.apply(got[0], xd, pd.key_buffer, pd.value_buffer, *idx, slots[0], pd.a_scaling)
+        else:
+            one.apply_multi(got, xd, pd.key_buffer, pd.value_buffer, *idx, slots, pd.a_scaling)
+        for i in range(n_targets):
+            ref = O.lora_op(y0[i], x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids,
+                            slots[i], pool.a_scaling, n_slots=n_slots)
+            assert_parity(got[i].cpu(), ref, what + f" target {i} rep {rep}")
+            none = (ids < 0)
+            assert torch.equal(got[i].cpu()[none], y0[i][none]), what + ": rows without an adapter changed"
+    # bit-identical to two launches wherever the library kept the requested split (a multi-target call may cut
+    # ksplit so that ksplit * targets <= 16; then the summation order differs and only the tolerance holds)
+    if one.ksplit * n_targets <= 16:
+        want = [y.to(dev) for y in y0]
+        if n_targets == 1:
+            two.apply(want[0], xd, pd.key_buffer, pd.value_buffer, *idx, slots[0], pd.a_scaling)
+        else:
+            two.apply_multi(want, xd, pd.key_buffer, pd.value_buffer, *idx, slots, pd.a_scaling)
+        for i in range(n_targets):
+            assert torch.equal(got[i], want[i]), what + f": target {i} differs from the two-launch op"
+
+
+@pytest.mark.parametrize("ks", [4, 5])
+def test_items_the_device_cannot_hold_from_the_start(dev, ks):
+    """64 tiles of one token each at 4096 -> 4096: with 5 K chunks the grid is larger than what the device
+    holds at once, so the last tiles' expand items start late by construction and must not trust stamps;
+    with 4 it just fits.  Either way the result is the two-launch op's."""
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(77)
+    A, T, h = 64, 64, 4096
+    pool = W.make_pool([16] * A, h, h, dtype, g, True, std=0.05)
+    ids = torch.randperm(A, generator=g)
+    x = torch.randn(T, h, generator=g).to(dtype)
+    y0 = torch.randn(T, h, generator=g).to(dtype)
+    pd = pool.to(dev)
+    idx = (pd.a_start, pd.a_len, pd.a_loc)
+    one = LoraPlan(ids.to(dev), pd.a_start, pd.a_len, 16, hidden=h, one_launch=True, ksplit=ks)
+    two = LoraPlan(ids.to(dev), pd.a_start, pd.a_len, 16, hidden=h, one_launch=False, bm_shrink=16, bm_expand=16,
+                   ksplit=ks, reduce_in_expand=True)
+    for rep in range(3):
+        a, b = y0.to(dev), y0.to(dev)
+        one.apply(a, x.to(dev), pd.key_buffer, pd.value_buffer, *idx, 1, pd.a_scaling)
+        two.apply(b, x.to(dev), pd.key_buffer, pd.value_buffer, *idx, 1, pd.a_scaling)
+        assert torch.equal(a, b), f"rep {rep}"
+    ref = O.lora_op(y0, x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, 1,
+                    pool.a_scaling)
+    assert_parity(a.cpu(), ref, "late items")
+
+
+def test_one_launch_request_on_a_large_batch_runs_as_two_launches(dev):
+    """A batch whose grid is far larger than the device is not run through the one-launch kernel (the library
+    decides per call); the request is honoured with the same bits."""
+    w = W.config3(hidden=512, mlp=1024, len_div=2, n_decode=64, targets=("q",))
+    wd = w.to(dev)
+    t = wd.target("q"); p = t.pool
+    R = max(p.ranks)
+    one, two = _pair(wd, "q", R, 512, 4)
+    a, b = wd.y0["q"].clone(), wd.y0["q"].clone()
+    one.apply(a, wd.x[512], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
+    two.apply(b, wd.x[512], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
+    assert torch.equal(a, b)

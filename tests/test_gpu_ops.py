@@ -239,10 +239,10 @@ def test_edge_cases_empty_and_no_adapter(dev):
                          p2.a_scaling, n_slots=n_slots)
         assert_parity(yy.cpu(), want, f"n_slots={n_slots}")
         yy = y2.to(dev)
-        plan16 = LoraPlan(ids2.to(dev), p2d.a_start, p2d.a_len, 32, n_slots=n_slots, hidden=256, bm_shrink=16)
-        plan16.apply_fused(yy, x2.to(dev), p2d.key_buffer, p2d.value_buffer, p2d.a_start, p2d.a_len, p2d.a_loc, slot,
-                           p2d.a_scaling)
-        assert_parity(yy.cpu(), want, f"fused n_slots={n_slots}")
+        plan16 = LoraPlan(ids2.to(dev), p2d.a_start, p2d.a_len, 32, n_slots=n_slots, hidden=256, one_launch=True)
+        plan16.apply(yy, x2.to(dev), p2d.key_buffer, p2d.value_buffer, p2d.a_start, p2d.a_len, p2d.a_loc, slot,
+                     p2d.a_scaling)
+        assert_parity(yy.cpu(), want, f"one launch n_slots={n_slots}")
 
 
 def test_plan_reuse_across_drop_in_calls(dev):

@@ -8,7 +8,7 @@ Modules mirror the reference's import points:
 * ``valora_amd.lora_prefill.lora_get_qkvo_fwd_{shrink,expand}``
                                               <- ``valora.models.peft.triton_kernel.lora.lora_prefill``
 * ``valora_amd.segments``                     <- ``set_sgmm_args`` / ``count_consecutive_requests``
-* ``valora_amd.plan.LoraPlan``                once-per-batch plan + fused shrink/expand
+* ``valora_amd.plan.LoraPlan``                once-per-batch plan + shrink/expand in one call
 """
 __version__ = "0.1.0"
 

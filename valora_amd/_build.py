@@ -14,7 +14,7 @@ from typing import List
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
-SOURCES = ["api.hip", "plan.hip", "shrink.hip", "expand.hip", "fused.hip", "pool.hip", "merge.hip"]
+SOURCES = ["api.hip", "plan.hip", "shrink.hip", "expand.hip", "decode.hip", "pool.hip", "merge.hip"]
 LIB_PATH = os.path.join(HERE, "libmlora.so")
 
 HIPCC_FLAGS = [

@@ -17,14 +17,14 @@ LIB_PATH = os.path.join(_HERE, "libmlora.so")
 
 MLORA_F16, MLORA_BF16 = 0, 1
 SHRINK_OVERWRITE, SHRINK_ZERO_PAD, SHRINK_ACCUMULATE = 0, 1, 2
-REDUCE_IN_EXPAND = 1
+REDUCE_IN_EXPAND, ONE_LAUNCH, ONE_LAUNCH_NO_WAIT = 1, 2, 4
 
 # every symbol include/mlora.h declares
 SYMBOLS = [
-    "mlora_last_error", "mlora_version", "mlora_plan_bytes", "mlora_scratch_bytes",
+    "mlora_last_error", "mlora_version", "mlora_plan_bytes", "mlora_scratch_bytes", "mlora_one_launch_scratch_bytes",
     "mlora_workspace_bytes", "mlora_build_plan", "mlora_count_consecutive",
     "mlora_ids_from_segments", "mlora_ids_from_requests", "mlora_shrink", "mlora_expand", "mlora_lora_apply",
-    "mlora_lora_apply_multi", "mlora_lora_fused", "mlora_dispatch_bgmv", "mlora_dispatch_bgmv_static",
+    "mlora_lora_apply_multi", "mlora_dispatch_bgmv", "mlora_dispatch_bgmv_static",
     "mlora_dispatch_sgmm", "mlora_prefill_shrink", "mlora_prefill_expand",
     "mlora_pool_alloc", "mlora_pool_alloc_contiguous", "mlora_pool_free", "mlora_pool_fill",
     "mlora_pool_scatter_rows", "mlora_pool_gather_rows", "mlora_index_compact", "mlora_merge_adapter",
@@ -63,11 +63,12 @@ def lib():
     L = ctypes.CDLL(LIB_PATH)
     L.mlora_last_error.restype = c_char_p
     L.mlora_version.restype = c_int
-    for n in ("mlora_plan_bytes", "mlora_scratch_bytes", "mlora_workspace_bytes"):
+    for n in ("mlora_plan_bytes", "mlora_scratch_bytes", "mlora_workspace_bytes", "mlora_one_launch_scratch_bytes"):
         getattr(L, n).restype = c_size_t
     L.mlora_plan_bytes.argtypes = [c_int64, c_int64]
     L.mlora_scratch_bytes.argtypes = [c_int64, c_int64, c_int32]
     L.mlora_workspace_bytes.argtypes = [c_int64, c_int64, c_int64]
+    L.mlora_one_launch_scratch_bytes.argtypes = [c_int64, c_int64, c_int64, c_int32, c_int32]
     L.mlora_build_plan.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_int64, c_void_p, c_void_p,
                                    c_int64, c_int32, c_int32, c_int32]
     L.mlora_count_consecutive.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
@@ -86,8 +87,6 @@ def lib():
     L.mlora_lora_apply_multi.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_size_t, c_void_p, c_int64, c_int64,
                                          c_int64, c_int64, POINTER(Pool), c_int32, POINTER(Target), c_void_p,
                                          c_int32, c_int32, c_int]
-    L.mlora_lora_fused.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
-                                   POINTER(Pool), POINTER(Pool), c_int32, c_void_p, c_int32, c_int]
     L.mlora_dispatch_bgmv.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,
                                       c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t]
     L.mlora_dispatch_bgmv_static.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,
@@ -113,7 +112,7 @@ def lib():
                                       c_void_p]
     L.mlora_merge_adapter.argtypes = [c_void_p, POINTER(c_void_p), POINTER(c_int32), c_int32, c_int64, c_int64, c_int64,
                                       POINTER(Pool), POINTER(Pool), c_int64, c_int64, ctypes.c_float, c_int32, c_int]
-    for n in SYMBOLS[5:]:  # everything after the size queries returns a status
+    for n in SYMBOLS[6:]:  # everything after the size queries returns a status
         getattr(L, n).restype = c_int
     _lib = L
     return L

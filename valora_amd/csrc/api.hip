@@ -27,6 +27,13 @@ int check_launch(const char *what) {
 }
 
 int expand_bn();
+int decode_bn();
+
+// Polls of a tile's "ready" word before an expand item of the one-launch op stops waiting and computes the
+// tile's partials itself.  A poll is one memory round trip plus a short sleep (about a microsecond), the shrink
+// items it waits for run for a few microseconds: the bound is far above anything a healthy launch needs and
+// only limits how long a workgroup can wait when its producers have not been scheduled.
+constexpr int ONE_LAUNCH_SPIN_LIMIT = 1024;
 
 namespace {
 
@@ -151,6 +158,16 @@ size_t mlora_plan_bytes(int64_t T, int64_t n_adapters) {
 size_t mlora_scratch_bytes(int64_t T, int64_t max_rank, int32_t ksplit) {
   if (T < 0 || max_rank < 0 || ksplit < 1) return 0;
   return scratch_bytes(T, max_rank, ksplit);
+}
+
+size_t mlora_one_launch_scratch_bytes(int64_t T, int64_t n_adapters, int64_t max_rank, int32_t ksplit,
+                                      int32_t n_targets) {
+  if (T < 0 || n_adapters < 0 || max_rank < 0 || n_targets < 1) return 0;
+  if (ksplit < 2) ksplit = 2;
+  if (ksplit * n_targets > DECODE_MAX_PRODUCERS) ksplit = DECODE_MAX_PRODUCERS / n_targets;
+  const int64_t rp = partial_stride(max_rank);
+  return (size_t)align_up(T * rp * 2, 256) +
+         4 * decode_partial_floats(tiles_upper(T, n_adapters, 16), n_targets, ksplit, rp);
 }
 
 size_t mlora_workspace_bytes(int64_t T, int64_t n_adapters, int64_t max_rank) {
@@ -339,6 +356,16 @@ int mlora_lora_apply(void *stream, const mlora_plan *plan, void *scratch, size_t
                      const mlora_pool *pool_a, const mlora_pool *pool_b, int32_t slot, const void *scales,
                      int32_t ksplit, int32_t flags, mlora_dtype dtype) {
   if (!plan) return fail(MLORA_ERR_INVALID, "lora_apply: plan is null");
+  if (flags & MLORA_ONE_LAUNCH) {
+    if (int rc = check_pool(pool_b, "lora_apply")) return rc;
+    mlora_target tg;
+    tg.y = y;
+    tg.w_b = pool_b->w;
+    tg.w_b_rows = pool_b->w_rows;
+    tg.slot = slot;
+    return mlora_lora_apply_multi(stream, plan, scratch, scratch_nbytes, x, T, h_in, h_out, max_rank, pool_a, 1, &tg,
+                                  scales, ksplit, flags, dtype);
+  }
   if (ksplit == 0) ksplit = default_ksplit(T, plan->n_adapters, plan->bm_shrink, h_in);
   if (int rc = mlora_shrink(stream, plan, scratch, scratch_nbytes, x, T, h_in, max_rank, pool_a, slot, ksplit, nullptr,
                             0, MLORA_SHRINK_OVERWRITE, 0, flags, dtype))
@@ -370,15 +397,38 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
       if (targets[j].y == targets[i].y) return fail(MLORA_ERR_INVALID, "lora_apply_multi: targets %d and %d share y", j, i);
   }
   if (ksplit == 0) ksplit = default_ksplit(T, plan->n_adapters, plan->bm_shrink, h_in);
+  const bool one_launch = (flags & MLORA_ONE_LAUNCH) != 0;
+  if (one_launch) {
+    if (plan->bm_shrink != 16 || plan->bm_expand != 16)
+      return fail(MLORA_ERR_NO_KERNEL, "lora_apply: the one-launch op needs a plan cut with bm_shrink = bm_expand = 16 (has %d / %d)",
+                  plan->bm_shrink, plan->bm_expand);
+    if (max_rank > 64) return fail(MLORA_ERR_NO_KERNEL, "lora_apply: max_rank=%lld > 64 uses the two-launch op", (long long)max_rank);
+    if (ksplit < 2) ksplit = 2;   // the hand-off carries fp32 K-chunk partials
+    if (ksplit * n_targets > DECODE_MAX_PRODUCERS) ksplit = DECODE_MAX_PRODUCERS / n_targets;
+  }
+  // The one-launch op is for grids the device holds (nearly) all at once: an item that starts late cannot
+  // take its tile's partials from the shrink items and computes them itself.  The grid is sized with an upper
+  // bound of the tile count, so some slack is allowed for workgroups that find no tile; a larger batch runs as
+  // two launches with the same ksplit, which gives the same bits.
+  bool one_launch_fits = false;
+  int decode_resident = 0;
+  if (one_launch) {
+    const int64_t groups8 = (tiles_upper(T, plan->n_adapters, 16) + 7) / 8 * 8;
+    const int64_t items = groups8 * ksplit * n_targets + groups8 * ((h_out + decode_bn() - 1) / decode_bn()) * n_targets;
+    decode_resident = decode_resident_workgroups((int)max_rank, dtype);
+    one_launch_fits = (flags & MLORA_ONE_LAUNCH_NO_WAIT) || (decode_resident > 0 && items * 4 <= (int64_t)decode_resident * 5);
+  }
+  const bool use_decode = one_launch && one_launch_fits;
   if (ksplit < 1 || ksplit > 64) return fail(MLORA_ERR_INVALID, "lora_apply_multi: ksplit=%d outside [1,64]", ksplit);
   const size_t per_target = scratch_bytes(T, max_rank, ksplit);
-  if (scratch_nbytes < per_target * (size_t)n_targets)
-    return fail(MLORA_ERR_WORKSPACE, "lora_apply_multi: scratch has %zu bytes, needs %zu", scratch_nbytes,
-                per_target * (size_t)n_targets);
+  const size_t scratch_need = use_decode ? mlora_one_launch_scratch_bytes(T, plan->n_adapters, max_rank, ksplit, n_targets)
+                                         : per_target * (size_t)n_targets;
+  if (scratch_nbytes < scratch_need)
+    return fail(MLORA_ERR_WORKSPACE, "lora_apply_multi: scratch has %zu bytes, needs %zu", scratch_nbytes, scratch_need);
   const PlanLayout L = plan_layout(plan->T, plan->n_adapters);
   const int64_t rp = partial_stride(max_rank);
   const int64_t v_bytes = align_up(T * rp * 2, 256);
-  const bool rie = ksplit > 1 && (flags & MLORA_REDUCE_IN_EXPAND);
+  const bool rie = one_launch || (ksplit > 1 && (flags & MLORA_REDUCE_IN_EXPAND));
   ShrinkArgs a;
   a.plan = static_cast<const int32_t *>(plan->dev);
   a.off_perm = L.off_perm;
@@ -404,11 +454,13 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
   for (int i = 0; i < MLORA_MAX_TARGETS; ++i) a.slots[i] = targets[i < n_targets ? i : 0].slot;
   a.out_tstride = (int64_t)(per_target / 2);
   a.partial_tstride = (int64_t)(per_target / 4);
-  if (int rc = launch_shrink((hipStream_t)stream, a, plan->bm_shrink, (int)max_rank,
-                             tiles_upper(T, plan->n_adapters, plan->bm_shrink), dtype))
-    return rc;
-  if (ksplit > 1 && !rie)
-    if (int rc = launch_shrink_reduce((hipStream_t)stream, a, dtype)) return rc;
+  if (!use_decode) {
+    if (int rc = launch_shrink((hipStream_t)stream, a, plan->bm_shrink, (int)max_rank,
+                               tiles_upper(T, plan->n_adapters, plan->bm_shrink), dtype))
+      return rc;
+    if (ksplit > 1 && !rie)
+      if (int rc = launch_shrink_reduce((hipStream_t)stream, a, dtype)) return rc;
+  }
 
   ExpandArgs e;
   e.plan = a.plan;
@@ -438,52 +490,25 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
   }
   e.v_tstride = a.out_tstride;
   e.partial_tstride = a.partial_tstride;
-  return launch_expand((hipStream_t)stream, e, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand), dtype);
-}
-
-int mlora_lora_fused(void *stream, const mlora_plan *plan, void *y, const void *x, int64_t T, int64_t h_in,
-                     int64_t h_out, int64_t max_rank, const mlora_pool *pool_a, const mlora_pool *pool_b,
-                     int32_t slot, const void *scales, int32_t replicas, mlora_dtype dtype) {
-  if (int rc = check_dtype(dtype, h_in, h_out)) return rc;
-  if (int rc = check_dims(T, h_in, max_rank, h_in, h_out, dtype)) return rc;
-  if (int rc = check_dims(T, h_out, max_rank, h_in, h_out, dtype)) return rc;
-  if (int rc = check_plan(plan, T, "lora_fused")) return rc;
-  if (int rc = check_pool(pool_a, "lora_fused")) return rc;
-  if (int rc = check_pool(pool_b, "lora_fused")) return rc;
-  if (plan->bm_shrink != 16)
-    return fail(MLORA_ERR_NO_KERNEL, "lora_fused: needs a plan built with bm_shrink=16 (has %d)", plan->bm_shrink);
-  if (max_rank > 64) return fail(MLORA_ERR_NO_KERNEL, "lora_fused: max_rank=%lld > 64 uses the two-launch path", (long long)max_rank);
-  if (T == 0) return MLORA_OK;
-  if (!y || !x || !scales) return fail(MLORA_ERR_INVALID, "lora_fused: null pointer");
-  if (!aligned16(y) || !aligned16(x)) return fail(MLORA_ERR_INVALID, "lora_fused: x and y must be 16-byte aligned");
-  if (slot < 0 || slot >= pool_a->n_slots || slot >= pool_b->n_slots)
-    return fail(MLORA_ERR_INVALID, "lora_fused: slot %d out of range", slot);
-  const int64_t tiles = tiles_upper(T, plan->n_adapters, 16);
-  const int64_t max_rep = (h_out + 63) / 64;
-  if (replicas == 0) {  // about 1.5 workgroups per compute unit
-    replicas = (int32_t)((384 + tiles - 1) / tiles);
+  if (use_decode) {
+    const int64_t tiles = tiles_upper(T, plan->n_adapters, 16);
+    int32_t *words = static_cast<int32_t *>(plan->dev);
+    DecodeArgs d;
+    d.s = a;
+    d.e = e;
+    d.done = reinterpret_cast<uint32_t *>(words + L.off_counters);
+    d.stamps = reinterpret_cast<uint32_t *>(words + L.off_stamps);
+    d.n_tiles = (int)tiles;
+    d.e.n_ochunks = (int)((h_out + decode_bn() - 1) / decode_bn());
+    d.n_producers = ksplit * n_targets;
+    d.n_consumers = d.e.n_ochunks * n_targets;
+    d.groups_per_chunk = decode_resident / (8 * (d.n_producers + d.n_consumers));
+    if (d.groups_per_chunk < 1) d.groups_per_chunk = 1;
+    d.spin_limit = (flags & MLORA_ONE_LAUNCH_NO_WAIT) ? 0 : ONE_LAUNCH_SPIN_LIMIT;
+    d.resident = decode_resident;
+    return launch_decode((hipStream_t)stream, d, (int)max_rank, dtype);
   }
-  if (replicas < 1) replicas = 1;
-  if (replicas > max_rep) replicas = (int32_t)max_rep;
-  const PlanLayout L = plan_layout(plan->T, plan->n_adapters);
-  FusedArgs a;
-  a.plan = static_cast<const int32_t *>(plan->dev);
-  a.off_perm = L.off_perm;
-  a.off_tiles = L.off_tiles_s;
-  a.y = static_cast<uint16_t *>(y);
-  a.x = static_cast<const uint16_t *>(x);
-  a.pa = pool_dev(pool_a);
-  a.pb = pool_dev(pool_b);
-  a.scales = static_cast<const uint16_t *>(scales);
-  a.T = (int)T;
-  a.h_in = (int)h_in;
-  a.h_out = (int)h_out;
-  a.kmax = (int)max_rank;
-  a.slot = slot;
-  a.tiles = (int)tiles;
-  a.tiles_pad = (int)align_up(tiles, 8);  // replicas of a tile land on the same XCD (workgroup id mod 8)
-  a.o_per_wg = (int)align_up((h_out + replicas - 1) / replicas, 64);
-  return launch_fused((hipStream_t)stream, a, (int)max_rank, replicas, dtype);
+  return launch_expand((hipStream_t)stream, e, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand), dtype);
 }
 
 // ---- one-call entry points ------------------------------------------------------------------------

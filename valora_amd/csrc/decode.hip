@@ -1,0 +1,414 @@
+// One-launch LoRA op for decode-like batches (few tokens per adapter) on gfx950:
+//
+//   y[t, o] = T( y[t, o] + scale_a * sum_j T(v[t, j]) * B_a[j, o] ),   v[t, j] = sum_k x[t, k] * A_a[j, k]
+//
+// At these sizes (tens of MB) two dependent launches cost more than the bytes: the expand's B fragments and
+// y rows cannot be requested before the shrink's grid has drained.  Here both halves are work items of ONE
+// grid.  Shrink items (tile, target, K chunk) compute their chunk's fp32 partial exactly like shrink_kernel
+// and leave it in the scratch buffer.  Expand items (tile, target, 512 output columns) request their B
+// fragments and y rows FIRST and only then wait for their tile's partials, so the wait overlaps loads they
+// need anyway.
+//
+// The hand-off stays inside one XCD.  The 8 XCDs of the device have an L2 each, and anything that has to be
+// visible across them goes to memory and back (measured here: 2.5 us per poll and 7 us to read a tile's
+// partials with device-scope loads; 0.5 us and 0.8 us inside an L2).  Workgroups are dealt to the XCDs round
+// robin by id, so the ids are laid out such that all items of tile t have id = t (mod 8): producer and
+// consumers of a tile share an L2, and the partials are plain stores and plain loads that meet there.
+// Nothing relies on the round-robin rule for correctness: a shrink item stamps its slot of the tile with
+// (the launch's tag, the XCD it runs on), an expand item only accepts stamps that carry its own tag and its
+// own XCD, and
+//   * an expand item polls a BOUNDED number of times; when the bound runs out -- its producers ran on another
+//     XCD, or were not scheduled, whatever the reason -- it computes the tile's partials itself, chunk by
+//     chunk with the shrink item's own code, so it gets the same bits and NO workgroup ever waits without
+//     limit: every wave of the grid reaches its end whatever the order, placement or residency of the
+//     workgroups;
+//   * the stamps are polled on the scalar path (scalar load that skips the scalar cache): a wave gets its
+//     vector-memory results strictly in order, so a vector poll would sit behind the B and y loads;
+//   * what tells a fresh stamp from one an earlier launch left behind is the tile's `done` word: every shrink
+//     item adds 1 to it when it has finished (device scope, nobody waits for the answer), and every item reads
+//     it when it starts and uses the value as the launch's tag.  All items that start before the tile's first
+//     shrink item finishes (microseconds later) read the same value, and it differs from every earlier
+//     launch's.  An item that starts later reads another value and matches nothing: correct, and slow.
+//     Therefore the items the device cannot hold from the start do not use the hand-off at all (see
+//     decode_kernel), and the host only picks this kernel for grids that (nearly) fit the device.
+//     Nothing is ever reset, so there is no moment at which a late writer could leave a stale "ready".
+//   * a tile's partials occupy whole 128-byte lines of their own, so no line is fetched before the tile is
+//     ready (a line shared with a neighbour tile could sit stale in a compute unit's L1).
+// Chunks are summed in index order, the same order as the two-launch path: results are bit-identical to it.
+// Launches that share a plan must not overlap in time (they share the scratch buffer and the words above).
+//
+// Reference semantics: valora/csrc/bgmv/bgmv_impl.cuh:14-148 (shrink) and :152-207 (expand).
+#include "kernel_common.h"
+#include "shrink_core.h"
+
+namespace mlora {
+
+namespace {
+
+constexpr int DEC_CH = 2;          // 256-column chunks per expand item (fewer, fatter items: the whole grid
+                                   // should be resident at once, a waiting item holds its slot)
+constexpr int DEC_BN = 256 * DEC_CH;   // outputs per expand item
+constexpr int DEC_WN = 64;         // outputs per wave and chunk
+constexpr int DEC_STAGE_LD = DEC_WN + 4;
+
+// device scope: visible to every compute unit, whichever XCD it sits on; the result is not asked for
+__device__ __forceinline__ void add_device(uint32_t *p, uint32_t v) {
+  (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// The 16 stamps of a tile as they are in this XCD's L2 right now, read on the scalar path: a scalar load with
+// glc skips the scalar cache, and its answer does not queue behind the wave's outstanding vector loads (the B
+// fragments and y rows requested just before), which come back strictly in order.
+typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ bool stamps_match(const uint32_t *stamps, int n, uint32_t want) {
+  u32x16 v;
+  asm volatile("s_load_dwordx16 %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(stamps) : "memory");
+  bool ok = true;
+#pragma unroll
+  for (int i = 0; i < DECODE_MAX_PRODUCERS; ++i) ok = ok && (i >= n || v[i] == want);
+  return ok;
+}
+// workgroup barrier that orders LDS traffic only: outstanding global loads stay in flight across it
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// which of the device's XCDs this wave runs on (bits 3:0 of the XCC_ID hardware register)
+__device__ __forceinline__ uint32_t xcd_id() { return (uint32_t)__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20); }
+
+__device__ __forceinline__ uint32_t stamp_of(uint32_t tag, uint32_t xcd) { return ((tag + 1u) << 4) | xcd; }
+
+// item id -> (role, tile, item of the tile).  A group is 8 consecutive tiles, a chunk as many groups as the
+// device holds at once.  Ids run chunk by chunk: first the chunk's shrink items, then its expand items, each as
+// (group, item, tile within the group) with the tile as the fast index, so the tile index mod 8 equals the id
+// mod 8 and the shrink items of the resident part of the grid are the first to be started.  The grid is sized
+// with an upper bound of the tile count; the tiles that do not exist are the last ones, so their items have
+// the highest ids of their chunk.
+struct ItemId {
+  bool shrink;
+  int tile, item;
+};
+__device__ __forceinline__ ItemId item_of(const DecodeArgs &a, int id) {
+  ItemId it;
+  const int per_group = 8 * (a.n_producers + a.n_consumers);
+  const int per_chunk = a.groups_per_chunk * per_group;
+  const int chunk = id / per_chunk, local = id - chunk * per_chunk;
+  const int n_shrink = a.groups_per_chunk * 8 * a.n_producers;
+  it.shrink = local < n_shrink;
+  const int l2 = it.shrink ? local : local - n_shrink;
+  const int per = it.shrink ? a.n_producers : a.n_consumers;
+  const int q8 = l2 >> 3, g = q8 / per;
+  it.item = q8 - g * per;
+  it.tile = (chunk * a.groups_per_chunk + g) * 8 + (l2 & 7);
+  return it;
+}
+
+// One workgroup = one work item.  The first `resident` workgroups are the ones the device holds from the start
+// (the hardware starts workgroups in id order); whatever has a higher id may start late, i.e. after shrink
+// items of its tile have finished and moved the tile's tag on.  Such an expand item does not look at stamps
+// at all but computes its tile's partials itself, and such a shrink item has nobody who would use its result
+// (a tile's expand items come after its shrink items) and does nothing.  With the ids running chunk by
+// chunk, these are the items of the tiles that do not exist, unless the batch is larger than the device.
+// 3 waves per SIMD = 3 workgroups per compute unit: an expand item keeps the B fragments and y rows of 512
+// columns in flight, a shrink item 8 K-steps of both operands.
+template <typename T, int NB>
+__global__ __launch_bounds__(256, 3) void decode_kernel(DecodeArgs a) {
+  using Tr = Traits<T>;
+  using vec8 = typename Tr::vec8;
+  constexpr int KB = (NB + 1) / 2;                  // 32-wide rank blocks of the expand
+  constexpr int STAGE_FLOATS = 4 * 16 * DEC_STAGE_LD;
+  constexpr int RED_FLOATS = 2 * NB * 256;          // cross-wave reduction of shrink_tile_to_lds
+  constexpr int VACC_FLOATS = 16 * NB * 16;         // a tile's summed chunks (give-up path)
+  static_assert(DECODE_MAX_PRODUCERS == 16, "stamps_match reads 16 stamps");
+  static_assert(RED_FLOATS + VACC_FLOATS <= STAGE_FLOATS, "the shrink buffers alias the expand's staging tile");
+  __shared__ __align__(16) float s_buf[STAGE_FLOATS];
+  __shared__ int32_t s_perm[16];
+  __shared__ int32_t s_ready;
+  float(*red)[NB * 256] = reinterpret_cast<float(*)[NB * 256]>(s_buf);
+  const int id = (int)blockIdx.x;
+  const bool on_time = id < a.resident;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rp = a.s.rp;
+  const int32_t *__restrict__ perm = a.s.plan + a.s.off_perm;
+
+  const ItemId it = item_of(a, id);
+  const bool shrink_item = it.shrink;
+  const int item = it.item, tile_idx = it.tile;
+  if (tile_idx >= a.n_tiles) return;
+  const int32_t *__restrict__ tile = a.s.plan + a.e.off_tiles + (int64_t)tile_idx * TILE_WORDS;
+  const int ad = tile[0], r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
+  if (cnt <= 0) return;   // records past the last tile are zero
+  if (shrink_item && !on_time) return;
+  // the launch's tag: what the tile's `done` word holds while none of this launch's shrink items has finished
+  const uint32_t want_stamp = stamp_of(a.done[tile_idx], xcd_id());
+  uint32_t *const stamps = a.stamps + (int64_t)tile_idx * DECODE_MAX_PRODUCERS;
+  // a tile's partials: [target][K chunk][16 rows][rp] floats, whole lines of the tile's own
+  float *const tile_partial = a.s.partial + (int64_t)tile_idx * a.n_producers * 16 * rp;
+
+  // ------------------------------------------------------------------ shrink item
+  if (shrink_item) {
+    const int z = item / a.s.ksplit, s = item - z * a.s.ksplit;
+    const int kbeg = s * a.s.kchunk;
+    const int kend = min(a.s.h_in, kbeg + a.s.kchunk);
+    shrink_tile_to_lds<T, 1, NB>(a.s.x, a.s.h_in, a.s.pool, a.s.slots[z], perm, r, pos0, cnt, astart, kbeg, kend, red);
+    if (wave == 0) {
+      // wave 0 alone writes the partial and then the stamp: no barrier, and nothing else of its own in flight
+      f32x4 *part = reinterpret_cast<f32x4 *>(tile_partial + (int64_t)item * 16 * rp);
+      const int quarter = rp >> 2;
+      for (int e = lane; e < 16 * quarter; e += 64) {
+        const int row = e / quarter, c4 = e - row * quarter;
+        const float *src = red[1] + row * (NB * 16) + 4 * c4;
+        part[e] = f32x4{src[0], src[1], src[2], src[3]};
+      }
+      // the partial must sit in the L2 before the stamp that announces it
+      wait_vmcnt<0>();
+      if (lane == 0) __hip_atomic_store(stamps + item, want_stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    } else if (tid == 64) {
+      add_device(a.done + tile_idx, 1u);
+    }
+    return;
+  }
+
+  // ------------------------------------------------------------------ expand item
+  const int z = item / a.e.n_ochunks, oc = item - z * a.e.n_ochunks;
+  const int rk = min(r, a.e.kmax);   // rank columns the narrow operand really has (bgmv_impl.cuh:167,186)
+  const int slot = a.e.slots[z];
+  uint16_t *const y = a.e.ys[z];
+  const uint16_t *const wB = a.e.ws[z];
+  const int64_t wB_rows = a.e.w_rows_t[z];
+  const int h_out = a.e.h_out;
+
+  const int lrow = lane & 15, kg = lane >> 4;
+  const int64_t base = (int64_t)astart + (int64_t)r * slot;
+  int o_wave[DEC_CH];
+#pragma unroll
+  for (int c = 0; c < DEC_CH; ++c) o_wave[c] = oc * DEC_BN + c * 256 + wave * DEC_WN;
+
+  // Everything that depends only on the tile record is requested first, in one round trip.  The set-up is
+  // kept to few instructions and free of branches: with every workgroup of the grid resident, the vector
+  // ALUs are what the first loads wait for.  Loads that have nothing to fetch read element 0 of their
+  // array instead of being skipped, and their result is dropped.
+  int my_perm = 0;
+  if (tid < cnt) my_perm = perm[pos0 + tid];
+  const float scale = Tr::to_float(a.e.scales[ad]);
+  const float inv_h_out = 1.0f / (float)h_out;
+  const uint32_t base32 = (uint32_t)(astart + r * slot), n_loc = (uint32_t)a.e.pool.a_loc_len;
+  const uint32_t step16 = 16u * (uint32_t)r;
+  const bool can_step = step16 < (uint32_t)h_out;     // workgroup-uniform
+  int64_t brow[DEC_CH][4][KB];
+  uint32_t boff[DEC_CH][4][KB];
+  bool bok[DEC_CH][4][KB];
+#pragma unroll
+  for (int c = 0; c < DEC_CH; ++c)
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const uint32_t j0 = (uint32_t)(kb * 32 + kg * 8);
+      BCursor cur = b_cursor((uint32_t)(o_wave[c] + lrow), (uint32_t)r, j0, (uint32_t)h_out, inv_h_out);
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) {
+        const int o = o_wave[c] + nb * 16 + lrow;
+        if (nb > 0) {
+          if (can_step) b_advance(cur, step16, (uint32_t)h_out);
+          else cur = b_cursor((uint32_t)o, (uint32_t)r, j0, (uint32_t)h_out, inv_h_out);
+        }
+        const uint32_t idx = base32 + cur.bin;
+        const bool ok = o < h_out && (int)j0 < rk && idx < n_loc;
+        brow[c][nb][kb] = a.e.pool.a_loc[ok ? idx : 0u];
+        boff[c][nb][kb] = cur.off;
+        bok[c][nb][kb] = ok;
+      }
+    }
+  if (tid < 16) s_perm[tid] = my_perm;
+  __syncthreads();
+
+  // B fragments and y rows: the loads the hand-off wait is hidden behind
+  u32x4 bfrag[DEC_CH][4][KB];
+#pragma unroll
+  for (int c = 0; c < DEC_CH; ++c)
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        const int64_t row = brow[c][nb][kb];
+        const bool ok = bok[c][nb][kb] && (uint64_t)row < (uint64_t)wB_rows;
+        const u32x4 got = load16(wB + (ok ? row * h_out + boff[c][nb][kb] : 0));
+        bfrag[c][nb][kb] = ok ? got : u32x4{0, 0, 0, 0};
+      }
+  const int rr0 = lane >> 3, c8 = (lane & 7) * 8;
+  u32x4 yv[DEC_CH][2];
+  uint16_t *yp[DEC_CH][2];
+  bool yok[DEC_CH][2];
+#pragma unroll
+  for (int c = 0; c < DEC_CH; ++c)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int row = rr0 + 8 * h;
+      yok[c][h] = (o_wave[c] + c8) < h_out && row < cnt;
+      yp[c][h] = y + (yok[c][h] ? (int64_t)s_perm[row] * h_out + o_wave[c] + c8 : 0);
+      yv[c][h] = load16(yp[c][h]);
+    }
+  // ---- bounded wait for the tile's stamps (one wave polls on the scalar path; the workgroup follows its
+  //      verdict without draining its loads)
+  if (wave == 0) {
+    int ok = 0;
+    for (int it = 0; on_time && it < a.spin_limit; ++it) {
+      if (stamps_match(stamps, a.n_producers, want_stamp)) { ok = 1; break; }
+      __builtin_amdgcn_s_sleep(2);
+    }
+    if (lane == 0) s_ready = ok;
+  }
+  lds_barrier();
+  const bool ready = s_ready != 0;
+
+  // ---- v fragment: rows = tokens (lrow), 8 consecutive rank elements per lane; chunks summed in index order
+  u32x4 vfrag[KB];
+  const bool pok = lrow < cnt;
+  if (ready) {
+    const float *part = tile_partial + (int64_t)z * a.e.ksplit * 16 * rp;
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int j0 = kb * 32 + kg * 8;
+      u32x4 v = {0, 0, 0, 0};
+      if (pok && j0 < rk) {
+        float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        const float *src0 = part + lrow * rp + j0;
+        for (int s0 = 0; s0 < a.e.ksplit; s0 += 4) {
+          f32x4 lo[4], hi[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const bool ok = s0 + u < a.e.ksplit;
+            const f32x4 *src = reinterpret_cast<const f32x4 *>(src0 + (int64_t)(s0 + u) * 16 * rp);
+            lo[u] = ok ? src[0] : f32x4{0.f, 0.f, 0.f, 0.f};
+            hi[u] = ok ? src[1] : f32x4{0.f, 0.f, 0.f, 0.f};
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { f[i] += lo[u][i]; f[4 + i] += hi[u][i]; }
+        }
+        v = pack8<T>(f);
+      }
+      vfrag[kb] = v;
+    }
+  } else {
+    // give-up path: the tile's chunks computed here, one after the other with the shrink item's own code
+    float *vacc = s_buf + RED_FLOATS;
+    for (int e = tid; e < VACC_FLOATS; e += 256) vacc[e] = 0.f;
+    const int slot_a = a.s.slots[z];
+    for (int s = 0; s < a.s.ksplit; ++s) {
+      const int kbeg = s * a.s.kchunk;
+      const int kend = min(a.s.h_in, kbeg + a.s.kchunk);
+      shrink_tile_to_lds<T, 1, NB>(a.s.x, a.s.h_in, a.s.pool, slot_a, perm, r, pos0, cnt, astart, kbeg, kend, red);
+      for (int e = tid; e < VACC_FLOATS; e += 256) vacc[e] += red[1][e];
+      __syncthreads();
+    }
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      const int j0 = kb * 32 + kg * 8;
+      u32x4 v = {0, 0, 0, 0};
+      if (pok && j0 < rk && j0 < NB * 16) {
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = vacc[lrow * (NB * 16) + j0 + i];
+        v = pack8<T>(f);
+      }
+      vfrag[kb] = v;
+    }
+    __syncthreads();   // vacc is about to be reused as the staging tile
+  }
+
+  // ---- delta blocks through the matrix cores, turned through a wave-private LDS tile for the y update
+  float(*stage)[DEC_STAGE_LD] = reinterpret_cast<float(*)[DEC_STAGE_LD]>(s_buf + wave * 16 * DEC_STAGE_LD);
+#pragma unroll
+  for (int c = 0; c < DEC_CH; ++c) {
+    if (o_wave[c] < h_out) {   // wave-uniform
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+          if (kb * 32 < rk) acc = Tr::mfma(as<vec8>(vfrag[kb]), as<vec8>(bfrag[c][nb][kb]), acc);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) stage[kg * 4 + i][nb * 16 + lrow] = acc[i];
+      }
+      // the tile is private to this wave and a wave's LDS operations execute in order: only the compiler
+      // has to be kept from moving the reads below over the writes above
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        if (yok[c][h]) {
+          const float *srow = &stage[rr0 + 8 * h][c8];
+          float f[8];
+          unpack8<T>(yv[c][h], f);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) f[i] += scale * srow[i];
+          store16(yp[c][h], pack8<T>(f));
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+
+}
+
+template <typename T>
+int launch_decode_t(hipStream_t st, const DecodeArgs &a, int nb, dim3 grid) {
+  switch (nb) {
+    case 1: hipLaunchKernelGGL((decode_kernel<T, 1>), grid, dim3(256), 0, st, a); break;
+    case 2: hipLaunchKernelGGL((decode_kernel<T, 2>), grid, dim3(256), 0, st, a); break;
+    case 4: hipLaunchKernelGGL((decode_kernel<T, 4>), grid, dim3(256), 0, st, a); break;
+    default: return fail(MLORA_ERR_NO_KERNEL, "one-launch op: ranks above 64 use the two-launch path");
+  }
+  return check_launch("decode_kernel");
+}
+
+}  // namespace
+
+int decode_bn() { return DEC_BN; }
+
+// How many workgroups of decode_kernel the current device can hold at the same time (0 if the runtime cannot
+// tell).  The one-launch op is only used for grids that fit: an item that starts after its tile's shrink
+// items have finished falls back to computing the partials itself, which is correct and slow.
+int decode_resident_workgroups(int max_rank, mlora_dtype dt) {
+  int nb = (max_rank + 15) / 16;
+  nb = nb <= 1 ? 0 : nb <= 2 ? 1 : 2;
+  static int cached[64][2][3];   // [device][dtype][rank class], 0 = not asked yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  int &slot = cached[dev][dt == MLORA_F16 ? 0 : 1][nb];
+  if (slot > 0) return slot;
+  const void *fn = nullptr;
+  if (dt == MLORA_F16)
+    fn = nb == 0 ? (const void *)decode_kernel<_Float16, 1> : nb == 1 ? (const void *)decode_kernel<_Float16, 2>
+                                                                      : (const void *)decode_kernel<_Float16, 4>;
+  else
+    fn = nb == 0 ? (const void *)decode_kernel<__bf16, 1> : nb == 1 ? (const void *)decode_kernel<__bf16, 2>
+                                                                    : (const void *)decode_kernel<__bf16, 4>;
+  int per_cu = 0, cus = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, 0) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (per_cu <= 0 || cus <= 0) return 0;
+  slot = per_cu * cus;
+  return slot;
+}
+
+// floats of scratch the one-launch op needs for its partials: [tile][target][K chunk][16][rp]
+size_t decode_partial_floats(int64_t n_tiles, int n_targets, int ksplit, int64_t rp) {
+  return (size_t)n_tiles * (size_t)n_targets * (size_t)ksplit * 16u * (size_t)rp;
+}
+
+int launch_decode(hipStream_t st, const DecodeArgs &a, int max_rank, mlora_dtype dt) {
+  int nb = (max_rank + 15) / 16;
+  nb = nb <= 1 ? 1 : nb <= 2 ? 2 : nb <= 4 ? 4 : 8;
+  if (a.n_tiles <= 0) return MLORA_OK;
+  if (a.n_producers > DECODE_MAX_PRODUCERS)
+    return fail(MLORA_ERR_NO_KERNEL, "one-launch op: ksplit * targets = %d exceeds %d", a.n_producers, DECODE_MAX_PRODUCERS);
+  // whole chunks: the ids of a chunk that has fewer groups than the others still span a whole chunk
+  const int64_t groups = (a.n_tiles + 7) / 8;
+  const int64_t chunks = (groups + a.groups_per_chunk - 1) / a.groups_per_chunk;
+  const int64_t total = chunks * a.groups_per_chunk * 8 * ((int64_t)a.n_producers + a.n_consumers);
+  if (total > 0x7fffffff) return fail(MLORA_ERR_NO_KERNEL, "one-launch op: grid too large");
+  dim3 grid((unsigned)total);
+  return dt == MLORA_F16 ? launch_decode_t<_Float16>(st, a, nb, grid) : launch_decode_t<__bf16>(st, a, nb, grid);
+}
+
+}  // namespace mlora

@@ -69,6 +69,7 @@ __global__ __launch_bounds__(256, expand_min_waves(KB, PARTIAL)) void expand_ker
   int my_perm = 0;
   if (tid < cnt) my_perm = p.plan[p.off_perm + pos0 + tid];
   const float scale = Tr::to_float(p.scales[a]);
+  const float inv_h_out = 1.0f / (float)p.h_out;
   int64_t brow[4][KB];
   uint32_t boff[4][KB];
 #pragma unroll
@@ -81,8 +82,8 @@ __global__ __launch_bounds__(256, expand_min_waves(KB, PARTIAL)) void expand_ker
       boff[nb][kb] = 0;
       if (o < p.h_out && j0 < rk) {
         const uint32_t flat = (uint32_t)o * (uint32_t)r + (uint32_t)j0;   // < 2^16 * 2^7
-        const uint32_t bin = flat / (uint32_t)p.h_out;
-        boff[nb][kb] = flat - bin * (uint32_t)p.h_out;
+        uint32_t bin;
+        divmod24(flat, (uint32_t)p.h_out, inv_h_out, bin, boff[nb][kb]);
         const int64_t idx = base + bin;
         if (idx >= 0 && idx < p.pool.a_loc_len) brow[nb][kb] = p.pool.a_loc[idx];
       }

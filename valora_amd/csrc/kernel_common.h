@@ -54,6 +54,43 @@ __device__ __forceinline__ void lds_write16(uint32_t off, u32x4 v) {
 // makes v "produced here" for the compiler, so nothing that uses it moves above a preceding wait
 __device__ __forceinline__ void pin(u32x4 &v) { asm volatile("" : "+v"(v)); }
 
+// q = n / d and rem = n % d for n < 2^24 (exact in fp32) from a reciprocal computed once: the float estimate of
+// the quotient is off by at most one.  An integer division by a run-time divisor costs some 35 vector
+// instructions, and the kernels' address set-up does several per lane before the first load can be issued.
+__device__ __forceinline__ void divmod24(uint32_t n, uint32_t d, float inv_d, uint32_t &q, uint32_t &rem) {
+  q = (uint32_t)((float)n * inv_d);
+  int32_t m = (int32_t)(n - q * d);
+  if (m < 0) {
+    q -= 1u;
+    m += (int32_t)d;
+  } else if (m >= (int32_t)d) {
+    q += 1u;
+    m -= (int32_t)d;
+  }
+  rem = (uint32_t)m;
+}
+
+// Walks the B operand of the expand.  A slot's B block is r pool rows that, concatenated, hold [h_out, r]
+// row-major: the 8 rank elements [j0, j0 + 8) of output column o start at flat offset o*r + j0, i.e. in the
+// slot's pool row number `bin` at element `off`.  Outputs 16 apart are 16*r elements apart, so after one
+// division the cursor moves on with an add and a compare.
+struct BCursor {
+  uint32_t bin, off;
+};
+__device__ __forceinline__ BCursor b_cursor(uint32_t o, uint32_t r, uint32_t j0, uint32_t h_out, float inv_h_out) {
+  BCursor c;
+  divmod24(o * r + j0, h_out, inv_h_out, c.bin, c.off);   // o < 2^16, r <= 2^7
+  return c;
+}
+// `step` elements further on; step < h_out
+__device__ __forceinline__ void b_advance(BCursor &c, uint32_t step, uint32_t h_out) {
+  c.off += step;
+  if (c.off >= h_out) {
+    c.off -= h_out;
+    c.bin += 1u;
+  }
+}
+
 template <typename T>
 struct Traits;
 

@@ -10,12 +10,13 @@ namespace mlora {
 
 // ---- plan buffer layout (int32 words) ------------------------------------------------------
 //   hdr[32] | perm[T] | padapter[T] | prank[T] | tiles_s[max_tiles][8] | tiles_e[max_tiles][8]
-//   | counters[max_tiles] | scratch: cnt[A] gstart[A] toff_s[A] toff_e[A]
+//   | done[max_tiles] | stamps[max_tiles][DECODE_MAX_PRODUCERS] | scratch: cnt[A] gstart[A] toff_s[A] toff_e[A]
 // perm[p]     token index at sorted position p (tokens grouped by adapter, original order kept
 //             inside a group); positions >= hdr[H_NACTIVE] are unused
 // padapter[p] adapter of position p;  prank[p] its rank
 // tile        {adapter, rank, first position, token count, a_start[adapter], 0, 0, 0}
-// counters[i] reserved (zeroed by the plan kernel)
+// done, stamps  the hand-off words of the one-launch op (csrc/decode.hip): per tile a count of the shrink items
+//             that have finished on this plan, and one stamp per shrink item; zeroed by the plan kernel
 constexpr int HDR_WORDS = 32;
 constexpr int TILE_WORDS = 8;
 constexpr int32_t PLAN_MAGIC = 0x4d4c5241;
@@ -29,10 +30,11 @@ enum PlanErr { PERR_START_OVERFLOW = 1 };
 constexpr int64_t MAX_ADAPTERS = 8192;   // per-wave histograms live in LDS
 constexpr int64_t MAX_TOKENS = 1 << 22;
 constexpr int MAX_RANK = 128;
+constexpr int DECODE_MAX_PRODUCERS = 16;   // shrink items per tile (K chunks x targets) of the one-launch op
 
 struct PlanLayout {
   int64_t T, A, max_tiles;
-  int64_t off_perm, off_padapter, off_prank, off_tiles_s, off_tiles_e, off_counters, off_scratch, total_words;
+  int64_t off_perm, off_padapter, off_prank, off_tiles_s, off_tiles_e, off_counters, off_stamps, off_scratch, total_words;
 };
 
 static inline __host__ __device__ int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
@@ -48,7 +50,8 @@ static inline PlanLayout plan_layout(int64_t T, int64_t A) {
   L.off_tiles_s = align_up(L.off_prank + T, 8);
   L.off_tiles_e = L.off_tiles_s + L.max_tiles * TILE_WORDS;
   L.off_counters = L.off_tiles_e + L.max_tiles * TILE_WORDS;
-  L.off_scratch = align_up(L.off_counters + L.max_tiles, 8);
+  L.off_stamps = align_up(L.off_counters + L.max_tiles, 32);
+  L.off_scratch = align_up(L.off_stamps + L.max_tiles * DECODE_MAX_PRODUCERS, 8);
   L.total_words = L.off_scratch + 4 * A + 8;
   return L;
 }
@@ -110,18 +113,24 @@ struct ExpandArgs {
   int T, h_out, kmax, slot, n_ochunks;
 };
 
-struct FusedArgs {
-  const int32_t *plan;
-  int64_t off_perm, off_tiles;
-  uint16_t *y;
-  const uint16_t *x;
-  PoolDev pa, pb;
-  const uint16_t *scales;
-  int T, h_in, h_out, kmax, slot, tiles, tiles_pad, o_per_wg;   // tiles: records in the list; tiles_pad: rounded up to 8
-};
 
-int launch_fused(hipStream_t st, const FusedArgs &a, int max_rank, int replicas, mlora_dtype dt);
-int fused_bn();
+// one-launch op: shrink items and expand items of one grid (csrc/decode.hip)
+struct DecodeArgs {
+  ShrinkArgs s;               // partial-only shrink: s.partial, s.ksplit >= 2, tile height 16
+  ExpandArgs e;               // expand that sums the chunks: e.partial == s.partial, e.ksplit == s.ksplit
+  uint32_t *done;             // [tiles] shrink items finished on this plan so far (only ever counts up)
+  uint32_t *stamps;           // [tiles][DECODE_MAX_PRODUCERS] (launch tag, XCD) left by each shrink item
+  int n_tiles;                // upper bound of the tile count (records past the last tile are zero)
+  int groups_per_chunk;       // groups of 8 tiles whose items the device holds at once
+  int n_producers;            // shrink items per tile: ksplit * targets
+  int n_consumers;            // expand items per tile: column chunks * targets
+  int resident;               // workgroups the device holds at once: items with a higher id may start late
+  int spin_limit;             // polls of a tile's stamps before an expand item computes the partials itself
+};
+int launch_decode(hipStream_t st, const DecodeArgs &a, int max_rank, mlora_dtype dt);
+int decode_bn();
+int decode_resident_workgroups(int max_rank, mlora_dtype dt);   // workgroups of decode_kernel the current device holds at once
+size_t decode_partial_floats(int64_t n_tiles, int n_targets, int ksplit, int64_t rp);
 int launch_plan(hipStream_t st, int32_t *plan, const PlanLayout &L, const int64_t *ids,
                 const int64_t *a_start, const int64_t *a_len, int n_slots, int bm_s, int bm_e);
 size_t scratch_bytes(int64_t T, int64_t max_rank, int ksplit);

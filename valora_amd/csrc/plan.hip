@@ -57,7 +57,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
     int32_t *__restrict__ plan, const int64_t *__restrict__ ids, const int64_t *__restrict__ a_start,
     const int64_t *__restrict__ a_len, int T, int A, int n_slots, int bm_s, int bm_e, int W,
     int64_t off_perm, int64_t off_padapter, int64_t off_prank, int64_t off_tiles_s,
-    int64_t off_tiles_e, int64_t off_counters, int64_t off_scratch, int max_tiles) {
+    int64_t off_tiles_e, int64_t off_counters, int64_t off_scratch, int max_tiles, int n_flag_words) {
   __shared__ int32_t whist[HIST_WORDS];
   __shared__ int wsum[PLAN_WAVES + 1];
   __shared__ int s_maxrank;
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
   auto start_of = [&](int a) -> int64_t { return SMALL ? s_astart[a] : a_start[a]; };
 
   for (int i = tid; i < W * A; i += PLAN_THREADS) whist[i] = 0;
-  for (int i = tid; i < max_tiles; i += PLAN_THREADS) plan[off_counters + i] = 0;
+  for (int i = tid; i < n_flag_words; i += PLAN_THREADS) plan[off_counters + i] = 0;
   if (SMALL) {
     for (int a = tid; a < A; a += PLAN_THREADS) {
       const int64_t r = a_len[a] / n_slots;
@@ -316,11 +316,13 @@ int launch_plan(hipStream_t st, int32_t *plan, const PlanLayout &L, const int64_
   if (A <= PLAN_SMALL_A)
     hipLaunchKernelGGL(plan_kernel<true>, dim3(1), dim3(PLAN_THREADS), 0, st, plan, ids, a_start, a_len,
                        (int)L.T, A, n_slots, bm_s, bm_e, W, L.off_perm, L.off_padapter, L.off_prank,
-                       L.off_tiles_s, L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles);
+                       L.off_tiles_s, L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles,
+                       (int)(L.off_scratch - L.off_counters));
   else
     hipLaunchKernelGGL(plan_kernel<false>, dim3(1), dim3(PLAN_THREADS), 0, st, plan, ids, a_start, a_len,
                        (int)L.T, A, n_slots, bm_s, bm_e, W, L.off_perm, L.off_padapter, L.off_prank,
-                       L.off_tiles_s, L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles);
+                       L.off_tiles_s, L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles,
+                       (int)(L.off_scratch - L.off_counters));
   return check_launch("plan_kernel");
 }
 

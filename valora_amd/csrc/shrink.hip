@@ -15,6 +15,7 @@
 // Reference semantics: valora/csrc/bgmv/bgmv_impl.cuh:14-148 (per-token gather mat-vec with the
 // rank rows gathered through loc_indicies, fp32 accumulation, one T store per output).
 #include "kernel_common.h"
+#include "shrink_core.h"
 
 namespace mlora {
 
@@ -118,119 +119,16 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs args_in) {
   const int tile_idx = wg_tz / args_in.n_targets;
   const ShrinkArgs p = select_target(args_in, wg_tz - tile_idx * args_in.n_targets);
   const int s = blockIdx.x - wg_tz * p.ksplit;
-  using Tr = Traits<T>;
-  using vec8 = typename Tr::vec8;
   constexpr int NBLK = MB * NB;
   __shared__ float red[2][NBLK * 256];
 
   const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int lrow = lane & 15, kg = lane >> 4;
   const int32_t *__restrict__ perm = p.plan + p.off_perm;
-  const int64_t base = (int64_t)astart + (int64_t)r * p.slot;
-
-  const uint16_t *xp[MB];
-  bool xok[MB];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    const int row = mb * 16 + lrow;
-    xok[mb] = row < cnt;
-    const int t = xok[mb] ? perm[pos0 + row] : 0;
-    xp[mb] = p.x + (int64_t)t * p.h_in;
-  }
-  const uint16_t *wp[NB];
-  bool wok[NB];
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int j = nb * 16 + lrow;
-    const int64_t idx = base + j;
-    bool ok = (j < r) && idx >= 0 && idx < p.pool.a_loc_len;
-    int64_t row = ok ? p.pool.a_loc[idx] : 0;
-    ok = ok && row >= 0 && row < p.pool.w_rows;
-    wok[nb] = ok;
-    wp[nb] = p.pool.w + (ok ? row : 0) * p.h_in;
-  }
-
-  f32x4 acc[MB][NB];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
-
   const int kbeg = s * p.kchunk;
   const int kend = min(p.h_in, kbeg + p.kchunk);
-  // The trip count must be wave-uniform: MFMA ignores EXEC, so a lane that left the loop early
-  // would still feed its stale registers into the matrix core.  Lanes past the end load zeros.
-  constexpr int U = (MB + NB <= 2) ? 8 : (MB + NB <= 4) ? 4 : (MB + NB <= 8) ? 2 : 1;
-  for (int kb0 = kbeg + wave * 32; kb0 < kend; kb0 += 128 * U) {
-    u32x4 xa[U][MB], wb[U][NB];
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int k = kb0 + u * 128 + kg * 8;
-      const bool kok = k < kend;
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) xa[u][mb] = (xok[mb] && kok) ? load16(xp[mb] + k) : u32x4{0, 0, 0, 0};
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) wb[u][nb] = (wok[nb] && kok) ? load16(wp[nb] + k) : u32x4{0, 0, 0, 0};
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        if (nb * 16 < r) {
-#pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
-            acc[mb][nb] = Tr::mfma(as<vec8>(xa[u][mb]), as<vec8>(wb[u][nb]), acc[mb][nb]);
-        }
-      }
-    }
-  }
-
-  // cross-wave reduction (tree): waves 2,3 -> LDS, waves 0,1 add; wave 1 -> LDS, wave 0 adds.
-  if (wave >= 2) {
-    float *dst = red[wave - 2];
-#pragma unroll
-    for (int b = 0; b < NBLK; ++b)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) dst[(b * 4 + i) * 64 + lane] = acc[b / NB][b % NB][i];
-  }
-  __syncthreads();
-  if (wave < 2) {
-    const float *src = red[wave];
-#pragma unroll
-    for (int b = 0; b < NBLK; ++b)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[b / NB][b % NB][i] += src[(b * 4 + i) * 64 + lane];
-  }
-  __syncthreads();
-  if (wave == 1) {
-    float *dst = red[0];
-#pragma unroll
-    for (int b = 0; b < NBLK; ++b)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) dst[(b * 4 + i) * 64 + lane] = acc[b / NB][b % NB][i];
-  }
-  __syncthreads();
-  if (wave == 0) {
-    // wave 0 adds the last slot and leaves the finished tile in red[1], row-major
-    const float *src = red[0];
-    float *otile = red[1];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int b = mb * NB + nb;
-          const int row = mb * 16 + kg * 4 + i;  // C layout: column = lane%16, rows = 4*(lane/16)+i
-          const int col = nb * 16 + lrow;
-          otile[row * (NB * 16) + col] = acc[mb][nb][i] + src[(b * 4 + i) * 64 + lane];
-        }
-  }
-  __syncthreads();
+  shrink_tile_to_lds<T, MB, NB>(p.x, p.h_in, p.pool, p.slot, perm, r, pos0, cnt, astart, kbeg, kend, red);
   shrink_epilogue<T>(p, red[1], NB * 16, s, pos0, cnt, r, perm);
 }
 

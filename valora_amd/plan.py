@@ -22,10 +22,14 @@ class LoraPlan:
     def __init__(self, ids: torch.Tensor, a_start: torch.Tensor, a_len: torch.Tensor, max_rank: int,
                  n_slots: int = 4, hidden: int = 4096, bm_shrink: Optional[int] = None,
                  bm_expand: Optional[int] = None, ksplit: Optional[int] = None,
-                 reduce_in_expand: Optional[bool] = None):
+                 reduce_in_expand: Optional[bool] = None, one_launch: Optional[bool] = None,
+                 one_launch_no_wait: bool = False):
         """``ids``: int64 per-token adapter index (negative = no adapter); ``a_start`` / ``a_len``:
         the pool index (``a_len = n_slots * rank``); ``max_rank``: widest rank among the resident
-        adapters (the reference's ``max_lora_dim``, lora_unordered_batch_infer.py:181-182)."""
+        adapters (the reference's ``max_lora_dim``, lora_unordered_batch_infer.py:181-182).
+        ``one_launch``: shrink and expand as work items of one grid (decode-like batches; forces
+        16-token tiles, needs ``max_rank <= 64``); ``None`` takes the tile table's choice.
+        ``one_launch_no_wait`` makes every expand item take its give-up path (tests)."""
         if not ids.is_cuda:
             raise RuntimeError("ids must be a CUDA tensor")
         if ids.dtype != torch.long or a_start.dtype != torch.long or a_len.dtype != torch.long:
@@ -41,6 +45,15 @@ class LoraPlan:
         self.ksplit = max(1, cfg.ksplit if ksplit is None else ksplit)
         rie = cfg.reduce_in_expand if reduce_in_expand is None else reduce_in_expand
         self.flags = _lib.REDUCE_IN_EXPAND if rie else 0
+        self.one_launch = bool(cfg.one_launch if one_launch is None else one_launch)
+        if self.one_launch and (self.max_rank > 64 or bm_shrink not in (None, 16) or bm_expand not in (None, 16)):
+            if one_launch:
+                raise RuntimeError("No suitable kernel. the one-launch op needs 16-token tiles and max_rank <= 64")
+            self.one_launch = False
+        if self.one_launch:
+            self.bm_shrink = self.bm_expand = 16
+            self.ksplit = max(2, self.ksplit)
+            self.flags = _lib.REDUCE_IN_EXPAND | _lib.ONE_LAUNCH | (_lib.ONE_LAUNCH_NO_WAIT if one_launch_no_wait else 0)
         L = _lib.lib()
         nbytes = int(L.mlora_plan_bytes(self.T, self.n_adapters))
         self.buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
@@ -49,8 +62,14 @@ class LoraPlan:
         _lib.check(L.mlora_build_plan(_lib.current_stream(self.device), self.handle, _lib.ptr(ids.contiguous()),
                                       self.T, _lib.ptr(a_start), _lib.ptr(a_len), self.n_adapters, n_slots,
                                       self.bm_shrink, self.bm_expand))
-        sbytes = int(L.mlora_scratch_bytes(self.T, self.max_rank, self.ksplit))
-        self.scratch = torch.empty(sbytes, dtype=torch.uint8, device=self.device)
+        # room for a multi-target call from the start: the buffer is never replaced, so a HIP graph captured
+        # from this plan or work still queued on another stream keeps pointing at live memory
+        self.scratch_per_target = int(L.mlora_scratch_bytes(self.T, self.max_rank, self.ksplit))
+        nbytes = _lib.MAX_TARGETS * self.scratch_per_target
+        if self.one_launch:
+            nbytes = max(nbytes, max(int(L.mlora_one_launch_scratch_bytes(self.T, self.n_adapters, self.max_rank,
+                                                                          self.ksplit, n)) for n in (1, 2, 3, 4)))
+        self.scratch = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
 
     # -- introspection (synchronises; for tests and diagnostics) --------------------------------
     def header(self) -> dict:
@@ -135,9 +154,6 @@ class LoraPlan:
                 raise RuntimeError("all targets of one call must have the same output width")
         if scales.dtype != x.dtype:
             scales = scales.to(x.dtype)
-        need = n * int(_lib.lib().mlora_scratch_bytes(self.T, self.max_rank, self.ksplit))
-        if self.scratch.numel() < need:
-            self.scratch = torch.empty(need, dtype=torch.uint8, device=self.device)
         pa = _lib.make_pool(key_buffer, a_start, a_len, a_loc, h_in, self.n_slots)
         tg = (_lib.Target * n)()
         for i in range(n):
@@ -146,20 +162,6 @@ class LoraPlan:
             _lib.current_stream(self.device), self.handle, _lib.ptr(self.scratch), self.scratch.numel(), _lib.ptr(x),
             self.T, h_in, h_out, self.max_rank, pa, n, tg, _lib.ptr(scales), int(self.ksplit), self.flags,
             _lib.dtype_code(x.dtype)))
-
-    def apply_fused(self, y: torch.Tensor, x: torch.Tensor, key_buffer: torch.Tensor, value_buffer: torch.Tensor,
-                    a_start: torch.Tensor, a_len: torch.Tensor, a_loc: torch.Tensor, slot: int,
-                    scales: torch.Tensor, replicas: int = 0) -> None:
-        """Same result as ``apply`` in a single launch (plan must have ``bm_shrink == 16``)."""
-        self._check(x, y, key_buffer, value_buffer)
-        if scales.dtype != x.dtype:
-            scales = scales.to(x.dtype)
-        h_in, h_out = x.size(1), y.size(1)
-        pa = _lib.make_pool(key_buffer, a_start, a_len, a_loc, h_in, self.n_slots)
-        pb = _lib.make_pool(value_buffer, a_start, a_len, a_loc, h_out, self.n_slots)
-        _lib.check(_lib.lib().mlora_lora_fused(
-            _lib.current_stream(self.device), self.handle, _lib.ptr(y), _lib.ptr(x), self.T, h_in, h_out,
-            self.max_rank, pa, pb, int(slot), _lib.ptr(scales), int(replicas), _lib.dtype_code(x.dtype)))
 
     def apply(self, y: torch.Tensor, x: torch.Tensor, key_buffer: torch.Tensor, value_buffer: torch.Tensor,
               a_start: torch.Tensor, a_len: torch.Tensor, a_loc: torch.Tensor, slot: int,

@@ -32,6 +32,7 @@ class TileConfig:
     ksplit: int      # K-chunks the shrink is split into (partials summed by the consumer)
     bm_expand: int   # tokens per expand tile: multiple of 16 up to 256
     reduce_in_expand: bool = False  # split-K chunks summed by the expand launch (small batches)
+    one_launch: bool = False        # shrink and expand as work items of one grid (decode-like batches, rank <= 64)
 
 
 def _bucket(v: int, buckets) -> int:
@@ -71,7 +72,7 @@ def _load() -> None:
             raw = json.load(f)
         for k, v in raw.get("entries", {}).items():
             _table[k] = TileConfig(int(v["bm_shrink"]), int(v["ksplit"]), int(v["bm_expand"]),
-                                   bool(v.get("reduce_in_expand", False)))
+                                   bool(v.get("reduce_in_expand", False)), bool(v.get("one_launch", False)))
         _hiddens[:] = sorted({int(k.split(":")[2]) for k in _table})
 
 
@@ -86,9 +87,10 @@ def lookup(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> TileCo
         cfg = _table.get(key(n_tokens, max_rank, near, n_adapters))
         if cfg is not None:
             cfg = TileConfig(cfg.bm_shrink, max(1, min(cfg.ksplit, hidden // 128)), cfg.bm_expand,
-                             cfg.reduce_in_expand and min(cfg.ksplit, hidden // 128) > 1)
+                             cfg.reduce_in_expand and min(cfg.ksplit, hidden // 128) > 1,
+                             cfg.one_launch and hidden >= 256)
     if cfg is None:
         return fallback(n_tokens, max_rank, hidden, n_adapters)
     if max_rank > 64 and cfg.bm_shrink == 64:     # ranks above 64 have no 64-token shrink tile
-        cfg = TileConfig(32, cfg.ksplit, cfg.bm_expand, cfg.reduce_in_expand)
+        cfg = TileConfig(32, cfg.ksplit, cfg.bm_expand, cfg.reduce_in_expand, False)
     return cfg
