@@ -5,9 +5,9 @@
 // memory (token rows of x, rank rows of the pool), which is exactly the per-lane layout
 // v_mfma_f32_16x16x32 wants: lane (row = lane%16, kgroup = lane/16) holds 8 consecutive K elements,
 // so every operand is a single 16-byte global load straight into the MFMA source registers -- no LDS
-// staging, no transposes.  The four waves interleave 64-element K-steps (whole 128-byte lines), so the
-// workgroup reads 512 contiguous bytes of every row per round, and several K-steps are loaded before any
-// is consumed (the kernel is latency bound: what counts is the number of 16-byte loads in flight per lane).
+// staging, no transposes.  The four waves interleave 32-element K-steps, so the workgroup reads 256
+// contiguous bytes of every row per round, and several K-steps are loaded before any is consumed
+// (the kernel is latency bound: what counts is the number of 16-byte loads in flight per lane).
 //
 // Reference semantics: valora/csrc/bgmv/bgmv_impl.cuh:14-148 (per-token gather mat-vec with the
 // rank rows gathered through loc_indicies, fp32 accumulation).
@@ -62,37 +62,28 @@ __device__ __forceinline__ void shrink_tile_to_lds(const uint16_t *__restrict__ 
 
   // The trip count must be wave-uniform: MFMA ignores EXEC, so a lane that left the loop early
   // would still feed its stale registers into the matrix core.  Lanes past the end load zeros.
-  //
-  // A wave's step covers 64 K elements = one whole 128-byte line of every row: lane (row, kgroup) loads the
-  // 32 contiguous bytes [kgroup*16, kgroup*16 + 16) of the step with two 16-byte loads and feeds the halves
-  // to two MFMAs (any assignment of K elements to MFMA slots is fine as long as both operands use the same
-  // one).  Asking for the two halves of a line from two different waves costs a second request per line.
-  constexpr int U = (MB + NB <= 2) ? 4 : (MB + NB <= 4) ? 2 : 1;     // 64-element steps in flight
-  for (int kb0 = kbeg + wave * 64; kb0 < kend; kb0 += 256 * U) {
-    u32x4 xa[U][2][MB], wb[U][2][NB];
+  // (Whole 128-byte lines per wave and step -- 64 K elements, two loads per lane -- measured the same to
+  // slightly slower than these half lines.)
+  constexpr int U = (MB + NB <= 2) ? 8 : (MB + NB <= 4) ? 4 : (MB + NB <= 8) ? 2 : 1;
+  for (int kb0 = kbeg + wave * 32; kb0 < kend; kb0 += 128 * U) {
+    u32x4 xa[U][MB], wb[U][NB];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
+      const int k = kb0 + u * 128 + kg * 8;
+      const bool kok = k < kend;
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int k = kb0 + u * 256 + kg * 16 + h * 8;
-        const bool kok = k < kend;
+      for (int mb = 0; mb < MB; ++mb) xa[u][mb] = (xok[mb] && kok) ? load16(xp[mb] + k) : u32x4{0, 0, 0, 0};
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) xa[u][h][mb] = (xok[mb] && kok) ? load16(xp[mb] + k) : u32x4{0, 0, 0, 0};
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) wb[u][h][nb] = (wok[nb] && kok) ? load16(wp[nb] + k) : u32x4{0, 0, 0, 0};
-      }
+      for (int nb = 0; nb < NB; ++nb) wb[u][nb] = (wok[nb] && kok) ? load16(wp[nb] + k) : u32x4{0, 0, 0, 0};
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
 #pragma unroll
-      for (int h = 0; h < 2; ++h) {
+      for (int nb = 0; nb < NB; ++nb) {
+        if (nb * 16 < r) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          if (nb * 16 < r) {
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-              acc[mb][nb] = Tr::mfma(as<vec8>(xa[u][h][mb]), as<vec8>(wb[u][h][nb]), acc[mb][nb]);
-          }
+          for (int mb = 0; mb < MB; ++mb)
+            acc[mb][nb] = Tr::mfma(as<vec8>(xa[u][mb]), as<vec8>(wb[u][nb]), acc[mb][nb]);
         }
       }
     }

@@ -99,6 +99,36 @@ def tune_shape(dev, n_tokens, n_adapters, rank, hidden, dtype=torch.float16, cop
     return {"bm_shrink": bm, "ksplit": ks, "bm_expand": best_e[1], "reduce_in_expand": bool(rie)}, best_e[0]
 
 
+def tune_one_launch(dev, n_tokens, n_adapters, rank, hidden, entry, dtype=torch.float16, copies=4):
+    """Does the one-launch op (shrink and expand items of one grid, 16-token tiles) beat the two-launch entry of
+    this shape?  Returns the entry to keep and both timings.  Only decode-like shapes qualify: rank <= 64 and a
+    grid the device holds at once (the library runs larger ones as two launches anyway)."""
+    ids, pool, x = synthetic_batch(n_tokens, n_adapters, rank, hidden, dtype, seed=n_tokens + n_adapters + rank)
+    ids, x, p = ids.to(dev), x.to(dev), pool.to(dev)
+    ys = [torch.zeros(ids.numel(), hidden, dtype=dtype, device=dev) for _ in range(copies)]
+    idx = (p.a_start, p.a_len, p.a_loc)
+
+    def op_us(**kw):
+        plan = LoraPlan(ids, p.a_start, p.a_len, rank, hidden=hidden, **kw)
+        return _time(lambda: [plan.apply(y, x, p.key_buffer, p.value_buffer, *idx, 0, p.a_scaling)
+                              for y in ys]) / copies
+
+    two = op_us(bm_shrink=entry["bm_shrink"], ksplit=entry["ksplit"], bm_expand=entry["bm_expand"],
+                reduce_in_expand=entry.get("reduce_in_expand", False), one_launch=False)
+    best = None
+    for ks in (4, 2, 3, 6, 8):
+        if ks * 128 > hidden:
+            continue
+        us = op_us(ksplit=ks, one_launch=True)
+        if best is None or us < 0.97 * best[0]:
+            best = (us, ks)
+    if best[0] < 0.97 * two:
+        return {"bm_shrink": 16, "ksplit": best[1], "bm_expand": 16, "reduce_in_expand": True, "one_launch": True}, two, best[0]
+    keep = dict(entry)
+    keep.pop("one_launch", None)
+    return keep, two, best[0]
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--overwrite", action="store_true")
@@ -107,6 +137,9 @@ def main():
     ap.add_argument("--adapters", type=int, nargs="+", default=[8, 32, 128])
     ap.add_argument("--ranks", type=int, nargs="+", default=list(tt.RANK_BUCKETS))
     ap.add_argument("--out", default=tt.TABLE_PATH)
+    ap.add_argument("--one-launch", action="store_true",
+                    help="revisit the existing entries of decode-like shapes (<= 1024 tokens, rank <= 64; the protected "
+                         "ones too) and mark those where the one-launch op is faster than the entry's two launches")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("tune_tiles needs a GPU")
@@ -117,6 +150,14 @@ def main():
     t0 = time.time()
     for hidden, n_tokens, n_adapters, rank in itertools.product(args.hidden, args.tokens, args.adapters, args.ranks):
         k = tt.key(n_tokens, rank, hidden, n_adapters)
+        if args.one_launch:
+            if k in entries and n_tokens <= 1024 and rank <= 64:
+                entries[k], two, one = tune_one_launch(dev, n_tokens, min(n_adapters, max(1, n_tokens)), rank, hidden,
+                                                       entries[k])
+                print(f"{k:24s} two launches {two:.1f} us, one launch {one:.1f} us -> {entries[k]}  "
+                      f"[{time.time() - t0:.0f} s]", flush=True)
+                torch.cuda.empty_cache()
+            continue
         if k in entries and (not args.overwrite or k in table.get("protected", [])):
             print(f"{k:24s} kept {entries[k]}", flush=True)
             continue
