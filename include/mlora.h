@@ -59,6 +59,14 @@ enum {
                                  testable; same results, slower)                                  */
 };
 
+/* What the kernels can vary per batch shape (see mlora_tile_lookup). */
+typedef struct {
+  int32_t bm_shrink;        /* tokens per shrink tile: 16, 32, 64 (direct loads) or 128 (LDS-staged)  */
+  int32_t ksplit;           /* K chunks the shrink is split into                                      */
+  int32_t bm_expand;        /* tokens per expand tile: multiple of 16 up to 256                       */
+  int32_t flags;            /* MLORA_REDUCE_IN_EXPAND | MLORA_ONE_LAUNCH                              */
+} mlora_tile_config;
+
 /* Pool + adapter index operands shared by all op entry points (device pointers).
  * Semantics: valora/server/router/model_infer/infer_adapter.py:14-17,128-148.            */
 typedef struct {
@@ -81,6 +89,8 @@ typedef struct {
   int64_t n_adapters;
   int32_t bm_shrink;        /* tile heights in tokens the two tile lists were cut with          */
   int32_t bm_expand;
+  int32_t n_slots;          /* slots per adapter of the index the plan was cut for; the op entry
+                               points reject a pool whose n_adapters or n_slots differ           */
 } mlora_plan;
 
 const char *mlora_last_error(void);
@@ -99,6 +109,20 @@ size_t mlora_one_launch_scratch_bytes(int64_t T, int64_t n_adapters, int64_t max
 /* Bytes of scratch the one-call entry points (dispatch_bgmv, dispatch_sgmm, prefill_*) need.
  * Replaces sgmm_tmp_size (atmm/valora/csrc/bgmv/bgmv_impl.cuh:128-132).                       */
 size_t mlora_workspace_bytes(int64_t T, int64_t n_adapters, int64_t max_rank);
+
+/* ---- tile selection ------------------------------------------------------------------------- */
+/* The tile configuration measured for this batch shape on MI355X: key (token bucket, rank bucket,
+ * hidden = wide dim of the shrink, adapter bucket); a width without entries takes those of the
+ * nearest measured width, anything else a rule.  Replaces shape_to_config / get_config_a /
+ * get_config_b (valora/models/peft/lora_unordered_batch_infer.py:25-172,216-236).  The one-call
+ * entry points use it themselves; callers of mlora_build_plan / mlora_lora_apply pass its answer
+ * on (bm_* to the plan, ksplit and flags to the op).                                          */
+int mlora_tile_lookup(int64_t n_tokens, int64_t max_rank, int64_t hidden, int64_t n_adapters,
+                      mlora_tile_config *out);
+/* The rule alone (what a shape without table entry gets): the counterpart of the reference's
+ * fixed fallback tuples (lora_unordered_batch_infer.py:224,235).                              */
+int mlora_tile_fallback(int64_t n_tokens, int64_t max_rank, int64_t hidden, int64_t n_adapters,
+                        mlora_tile_config *out);
 
 /* ---- index / segment builders ------------------------------------------------------------- */
 /* Adapter-grouped work tiles from per-token adapter ids (device int64[T]; an id outside
@@ -185,13 +209,21 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
                            const void *scales, int32_t ksplit, int32_t flags, mlora_dtype dtype);
 
 /* ---- the reference's entry points, one call each -------------------------------------------- */
+/* Each of the four takes an optional `plan`.  NULL: the call sorts the tokens and cuts the tiles
+ * itself, in `workspace` (mlora_workspace_bytes), with the tile table's configuration for the shape
+ * -- one extra launch per call.  The reference passes the same per-token ids to the 8 calls of a
+ * layer and to all layers of a forward pass (lora_unordered_batch_infer.py:946-1063), so a binding
+ * should build ONE plan per batch (mlora_tile_lookup + mlora_build_plan on the ids the calls would
+ * get; for the segment / per-request signatures on the output of mlora_ids_from_segments /
+ * mlora_ids_from_requests) and pass it to every call: then `indicies` / the segment operands are
+ * not read, an expand needs no workspace, and a shrink only mlora_scratch_bytes of it.          */
 /* dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, qkvo, lora_scales)
  * valora/csrc/lora_ops.cc:76-126.  Direction: h_in < h_out => expand, else shrink
  * (valora/csrc/bgmv/bgmv_impl.cuh:221).                                                       */
 int mlora_dispatch_bgmv(void *stream, void *y, const void *x, const mlora_pool *pool,
                         const int64_t *indicies, int64_t qkvo, const void *lora_scales, int64_t T,
                         int64_t h_in, int64_t h_out, mlora_dtype dtype, void *workspace,
-                        size_t workspace_bytes);
+                        size_t workspace_bytes, const mlora_plan *plan);
 
 /* mlora_dispatch_bgmv for callers that cannot allocate device memory and have no workspace to
  * bring: code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
@@ -218,7 +250,7 @@ int mlora_dispatch_sgmm(void *stream, void *y, const void *x, const mlora_pool *
                         const int64_t *output_counts, const int64_t *start_ids,
                         int64_t num_problems, int64_t T, int64_t h_in, int64_t h_out,
                         mlora_dtype dtype, int32_t shrink_mode, void *workspace,
-                        size_t workspace_bytes);
+                        size_t workspace_bytes, const mlora_plan *plan);
 
 /* lora_get_qkvo_fwd_shrink / lora_get_qkvo_fwd_expand
  * valora/models/peft/triton_kernel/lora/lora_prefill.py:139-163 / :105-135.                   */
@@ -226,12 +258,14 @@ int mlora_prefill_shrink(void *stream, void *o, const void *x, const mlora_pool 
                          const int32_t *b_start_loc, const int32_t *b_seq_len,
                          const int64_t *b_indicies, int64_t n_req, int64_t T, int64_t hidden,
                          int64_t o_stride, int64_t qkvo, int64_t max_rank, int64_t max_input_len,
-                         mlora_dtype dtype, void *workspace, size_t workspace_bytes);
+                         mlora_dtype dtype, void *workspace, size_t workspace_bytes,
+                         const mlora_plan *plan);
 int mlora_prefill_expand(void *stream, void *o, const void *x, const mlora_pool *pool,
                          const void *scale, const int32_t *b_start_loc, const int32_t *b_seq_len,
                          const int64_t *b_indicies, int64_t n_req, int64_t T, int64_t x_stride,
                          int64_t feat_out, int64_t qkvo, int64_t max_rank, int64_t max_input_len,
-                         mlora_dtype dtype, void *workspace, size_t workspace_bytes);
+                         mlora_dtype dtype, void *workspace, size_t workspace_bytes,
+                         const mlora_plan *plan);
 
 /* ---------------------------------------------------------------------------------------------
  * Adapter residency: the row allocator of the paged pool, loading / reading back an adapter's rows

@@ -58,13 +58,13 @@ def test_argument_validation_needs_no_gpu():
     assert rc == -2 and b"n_adapters=9000" in L.mlora_last_error()
     # dims outside what any kernel handles -> the reference's message shape
     pool = _lib.Pool(addr, 8, ctypes.addressof(a), ctypes.addressof(a), ctypes.addressof(a), 2, 2, 4)
-    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 0, addr, 4, 70000, 16, 0, addr, 1 << 15)
+    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 0, addr, 4, 70000, 16, 0, addr, 1 << 15, None)
     assert rc == -2 and L.mlora_last_error().startswith(b"No suitable kernel. h_in=70000 h_out=16 dtype=Half")
-    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 0, addr, 4, 4096, 12, 1, addr, 1 << 15)
+    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 0, addr, 4, 4096, 12, 1, addr, 1 << 15, None)
     assert rc == -2 and b"dtype=BFloat16" in L.mlora_last_error()
-    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 0, addr, 4, 4096, 16, 7, addr, 1 << 15)
+    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 0, addr, 4, 4096, 16, 7, addr, 1 << 15, None)
     assert rc == -2
-    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 5, addr, 4, 4096, 16, 0, addr, 1 << 15)
+    rc = L.mlora_dispatch_bgmv(None, addr, addr, pool, ctypes.addressof(ids), 5, addr, 4, 4096, 16, 0, addr, 1 << 15, None)
     assert rc == -1 and b"qkvo=5" in L.mlora_last_error()
 
 
@@ -83,6 +83,27 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libmlora.so")
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.lib()
+
+
+def test_tile_lookup_through_the_c_abi_agrees_with_the_json_table():
+    """Every entry of tile_table.json comes back from mlora_tile_lookup for a shape inside its bucket: the
+    table compiled into the library is the one the tuner wrote."""
+    import json
+    from valora_amd import tile_table as tt
+    L = _lib.lib()
+    with open(tt.TABLE_PATH) as f:
+        entries = json.load(f)["entries"]
+    assert len(entries) >= 100
+    for key, v in entries.items():
+        t, r, h, a = (int(p) for p in key.split(":"))
+        c = _lib.TileConfig()
+        assert L.mlora_tile_lookup(t, r, h, a, c) == 0
+        want_flags = (1 if v.get("reduce_in_expand") or v.get("one_launch") else 0) | (2 if v.get("one_launch") and r <= 64 else 0)
+        bm_s = 32 if (r > 64 and v["bm_shrink"] == 64) else v["bm_shrink"]
+        assert (c.bm_shrink, c.ksplit, c.bm_expand, c.flags) == (bm_s, v["ksplit"], v["bm_expand"], want_flags), key
+        assert tt.key(t, r, h, a) == key
+    c = _lib.TileConfig()
+    assert L.mlora_tile_lookup(-1, 16, 4096, 8, c) == -1 and L.mlora_tile_lookup(8, 16, 4096, 8, None) == -1
 
 
 def test_tile_table_lookup_and_fallback():

@@ -289,3 +289,105 @@ def test_plan_reuse_across_drop_in_calls(dev):
         assert (_plan_cache.hits, _plan_cache.misses) == (h1, m1)
     finally:
         _plan_cache.set_enabled(True)
+
+
+def test_one_call_entry_points_with_a_caller_held_plan(dev):
+    """What a binding that keeps ONE plan per batch does: mlora_tile_lookup + mlora_build_plan once, then every
+    dispatch_bgmv call of the layer with that plan -- no per-call sort, no workspace for the expand.  Same bits
+    as the calls that build their own plan."""
+    import ctypes
+    from valora_amd import _lib
+    L = _lib.lib()
+    dtype = torch.bfloat16
+    pool, ids, x, y0, v, R = _case(91, 300, 1024, 1024, (8, 16, 32, 16), dtype)
+    pd = pool.to(dev)
+    T, h = 300, 1024
+    stream = _lib.current_stream(dev)
+    ids_d, xd = ids.to(dev), x.to(dev)
+    pk = _lib.make_pool(pd.key_buffer, pd.a_start, pd.a_len, pd.a_loc, h, 4)
+    pv = _lib.make_pool(pd.value_buffer, pd.a_start, pd.a_len, pd.a_loc, h, 4)
+    cfg = _lib.TileConfig()
+    _lib.check(L.mlora_tile_lookup(T, R, h, 4, cfg))
+    buf = torch.empty(int(L.mlora_plan_bytes(T, 4)), dtype=torch.uint8, device=dev)
+    plan = _lib.Plan(_lib.ptr(buf), buf.numel())
+    _lib.check(L.mlora_build_plan(stream, plan, _lib.ptr(ids_d), T, _lib.ptr(pd.a_start), _lib.ptr(pd.a_len), 4, 4,
+                                  cfg.bm_shrink, cfg.bm_expand))
+    assert (plan.T, plan.n_adapters, plan.n_slots) == (T, 4, 4)
+    ws = torch.empty(int(L.mlora_workspace_bytes(T, 4, R)), dtype=torch.uint8, device=dev)
+    code = _lib.dtype_code(dtype)
+    out = {}
+    for held in (True, False):
+        delta = torch.full((T, R), 0.25, dtype=dtype, device=dev)
+        y = y0.to(dev)
+        p = plan if held else None
+        _lib.check(L.mlora_dispatch_bgmv(stream, _lib.ptr(delta), _lib.ptr(xd), pk, None if held else _lib.ptr(ids_d), 2,
+                                         _lib.ptr(pd.a_scaling), T, h, R, code, _lib.ptr(ws), ws.numel(), p))
+        # the expand on a caller-held plan takes no workspace at all
+        _lib.check(L.mlora_dispatch_bgmv(stream, _lib.ptr(y), _lib.ptr(delta), pv, None if held else _lib.ptr(ids_d), 2,
+                                         _lib.ptr(pd.a_scaling), T, R, h, code, None if held else _lib.ptr(ws),
+                                         0 if held else ws.numel(), p))
+        torch.cuda.synchronize()
+        out[held] = (delta.cpu(), y.cpu())
+    assert torch.equal(out[True][0], out[False][0]) and torch.equal(out[True][1], out[False][1])
+    want = O.lora_op(y0, x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, 2,
+                     pool.a_scaling)
+    assert_parity(out[True][1], want, "caller-held plan")
+    # a plan cut for another index is refused
+    other = _lib.make_pool(pd.key_buffer, pd.a_start[:3], pd.a_len[:3], pd.a_loc, h, 4)
+    rc = L.mlora_dispatch_bgmv(stream, _lib.ptr(y), _lib.ptr(xd), other, None, 2, _lib.ptr(pd.a_scaling), T, h, R, code,
+                               _lib.ptr(ws), ws.numel(), plan)
+    assert rc == -1 and b"plan was built for 4 adapters" in L.mlora_last_error()
+
+
+def test_plan_cache_hits_for_the_reference_call_patterns(dev):
+    """On the GPU, through the shims: the same tensors for all calls of a layer hit; fresh [1:] views of the
+    segment tensors hit; tensors created under inference_mode hit; a new ids tensor misses."""
+    from valora_amd import _plan_cache
+    from valora_amd.atmm_ops import dispatch_bgmv as dispatch_sgmm
+    from valora_amd.kernels import dispatch_bgmv
+    dtype = torch.float16
+    pool, ids, x, y0, v, R = _case(92, 120, 512, 512, (8, 16, 16), dtype)
+    pd = pool.to(dev)
+    idx = (pd.a_start, pd.a_len, pd.a_loc)
+    ids_d, xd = ids.to(dev), x.to(dev)
+    _plan_cache.clear()
+    h0, m0 = _plan_cache.hits, _plan_cache.misses
+    for layer in range(3):
+        for slot in range(3):
+            delta = torch.zeros(120, R, dtype=dtype, device=dev)
+            y = y0.to(dev)
+            dispatch_bgmv(delta, xd, pd.key_buffer, *idx, ids_d, slot, pd.a_scaling)
+            dispatch_bgmv(y, delta, pd.value_buffer, *idx, ids_d, slot, pd.a_scaling)
+    assert _plan_cache.misses - m0 == 1 and _plan_cache.hits - h0 == 17
+    # fresh offset views of the segment tensors with every call
+    oc, rc_, li, st = O.count_consecutive_requests(pool.a_len, ids)
+    P = len(oc)
+    t = lambda l: torch.tensor([9] + l + [1] * 4, dtype=torch.long, device=dev)
+    oc_d, st_d, rc_d, li_d = t(oc), t(st), t(rc_), t(li)
+    tmp = torch.zeros(60 * (P + 5), dtype=torch.int8, device=dev)
+    m1 = _plan_cache.misses
+    for _ in range(4):
+        delta = torch.zeros(120, R, dtype=dtype, device=dev)
+        dispatch_sgmm(delta, xd, pd.key_buffer, *idx, ids_d, 1, pd.a_scaling, oc_d[1:], rc_d[1:], li_d[1:], st_d[1:],
+                      tmp, P, 64, 32, 32, 32, 32, 32)
+    assert _plan_cache.misses - m1 == 1, "fresh views of the same segment tensors must reuse the plan"
+    want = O.sgmm_canonical(torch.zeros(120, R, dtype=dtype), x, pool.key_buffer, pool.a_start, pool.a_len, pool.a_loc, ids,
+                            1, pool.a_scaling, oc, st, P)
+    assert_parity(delta.cpu(), want, "sgmm through fresh views")
+    # inference tensors
+    with torch.inference_mode():
+        ids_i = ids.to(dev)
+        m2 = _plan_cache.misses
+        for _ in range(3):
+            delta = torch.zeros(120, R, dtype=dtype, device=dev)
+            dispatch_bgmv(delta, xd, pd.key_buffer, *idx, ids_i, 0, pd.a_scaling)
+        assert _plan_cache.misses - m2 == 1
+    # a new ids tensor with other contents
+    m3 = _plan_cache.misses
+    ids2 = torch.flip(ids, dims=(0,)).contiguous().to(dev)
+    delta = torch.zeros(120, R, dtype=dtype, device=dev)
+    dispatch_bgmv(delta, xd, pd.key_buffer, *idx, ids2, 0, pd.a_scaling)
+    assert _plan_cache.misses - m3 == 1
+    want = O.bgmv_shrink(torch.zeros(120, R, dtype=dtype), x, pool.key_buffer, pool.a_start, pool.a_len, pool.a_loc,
+                         torch.flip(ids, dims=(0,)), 0)
+    assert_parity(delta.cpu(), want, "new ids tensor")

@@ -27,7 +27,7 @@ def _pair(L, dev, pool, ids, x, narrow, v, y0, slot, dtype):
                                                   _lib.ptr(pool.a_scaling), T, h_in, h_out, code)
             else:
                 rc = L.mlora_dispatch_bgmv(stream, _lib.ptr(yy), _lib.ptr(xx), p, _lib.ptr(ids), slot,
-                                           _lib.ptr(pool.a_scaling), T, h_in, h_out, code, _lib.ptr(ws), ws.numel())
+                                           _lib.ptr(pool.a_scaling), T, h_in, h_out, code, _lib.ptr(ws), ws.numel(), None)
             _lib.check(rc)
         torch.cuda.synchronize()
         out.append((delta.cpu(), y.cpu()))

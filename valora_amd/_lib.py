@@ -22,7 +22,7 @@ REDUCE_IN_EXPAND, ONE_LAUNCH, ONE_LAUNCH_NO_WAIT = 1, 2, 4
 # every symbol include/mlora.h declares
 SYMBOLS = [
     "mlora_last_error", "mlora_version", "mlora_plan_bytes", "mlora_scratch_bytes", "mlora_one_launch_scratch_bytes",
-    "mlora_workspace_bytes", "mlora_build_plan", "mlora_count_consecutive",
+    "mlora_workspace_bytes", "mlora_tile_lookup", "mlora_tile_fallback", "mlora_build_plan", "mlora_count_consecutive",
     "mlora_ids_from_segments", "mlora_ids_from_requests", "mlora_shrink", "mlora_expand", "mlora_lora_apply",
     "mlora_lora_apply_multi", "mlora_dispatch_bgmv", "mlora_dispatch_bgmv_static",
     "mlora_dispatch_sgmm", "mlora_prefill_shrink", "mlora_prefill_expand",
@@ -46,7 +46,11 @@ MAX_TARGETS = 4
 
 class Plan(ctypes.Structure):
     _fields_ = [("dev", c_void_p), ("bytes", c_size_t), ("T", c_int64), ("n_adapters", c_int64),
-                ("bm_shrink", c_int32), ("bm_expand", c_int32)]
+                ("bm_shrink", c_int32), ("bm_expand", c_int32), ("n_slots", c_int32)]
+
+
+class TileConfig(ctypes.Structure):
+    _fields_ = [("bm_shrink", c_int32), ("ksplit", c_int32), ("bm_expand", c_int32), ("flags", c_int32)]
 
 
 _lib = None
@@ -69,6 +73,8 @@ def lib():
     L.mlora_scratch_bytes.argtypes = [c_int64, c_int64, c_int32]
     L.mlora_workspace_bytes.argtypes = [c_int64, c_int64, c_int64]
     L.mlora_one_launch_scratch_bytes.argtypes = [c_int64, c_int64, c_int64, c_int32, c_int32]
+    for n in ("mlora_tile_lookup", "mlora_tile_fallback"):
+        getattr(L, n).argtypes = [c_int64, c_int64, c_int64, c_int64, POINTER(TileConfig)]
     L.mlora_build_plan.argtypes = [c_void_p, POINTER(Plan), c_void_p, c_int64, c_void_p, c_void_p,
                                    c_int64, c_int32, c_int32, c_int32]
     L.mlora_count_consecutive.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
@@ -88,18 +94,18 @@ def lib():
                                          c_int64, c_int64, POINTER(Pool), c_int32, POINTER(Target), c_void_p,
                                          c_int32, c_int32, c_int]
     L.mlora_dispatch_bgmv.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,
-                                      c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t]
+                                      c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t, POINTER(Plan)]
     L.mlora_dispatch_bgmv_static.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,
                                              c_void_p, c_int64, c_int64, c_int64, c_int]
     L.mlora_dispatch_sgmm.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_int64,
                                       c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
-                                      c_int, c_int32, c_void_p, c_size_t]
+                                      c_int, c_int32, c_void_p, c_size_t, POINTER(Plan)]
     L.mlora_prefill_shrink.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_void_p,
                                        c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
-                                       c_int64, c_int, c_void_p, c_size_t]
+                                       c_int64, c_int, c_void_p, c_size_t, POINTER(Plan)]
     L.mlora_prefill_expand.argtypes = [c_void_p, c_void_p, c_void_p, POINTER(Pool), c_void_p, c_void_p,
                                        c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
-                                       c_int64, c_int64, c_int, c_void_p, c_size_t]
+                                       c_int64, c_int64, c_int, c_void_p, c_size_t, POINTER(Plan)]
     L.mlora_pool_alloc.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]
     L.mlora_pool_alloc_contiguous.argtypes = [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]
     L.mlora_pool_free.argtypes = [c_void_p, c_void_p, c_int64, c_void_p, c_int64]

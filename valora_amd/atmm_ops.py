@@ -72,7 +72,7 @@ def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, q
     _lib.check(_lib.lib().mlora_dispatch_sgmm(
         _lib.current_stream(x.device), _lib.ptr(y), _lib.ptr(x), pool, _lib.ptr(indicies), int(qkvo),
         _lib.ptr(lora_scales), _lib.ptr(output_counts.contiguous()), _lib.ptr(start_ids.contiguous()), P,
-        T, h_in, h_out, code, _SHRINK_MODE, _lib.ptr(ws), ws.numel()))
+        T, h_in, h_out, code, _SHRINK_MODE, _lib.ptr(ws), ws.numel(), None))
 
 
 dispatch_sgmm = dispatch_bgmv

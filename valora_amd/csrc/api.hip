@@ -60,6 +60,18 @@ int check_pool(const mlora_pool *pool, const char *who) {
   if (pool->n_slots < 1) return fail(MLORA_ERR_INVALID, "%s: n_slots must be >= 1", who);
   if (pool->n_adapters > MAX_ADAPTERS)
     return fail(MLORA_ERR_NO_KERNEL, "%s: more than %lld adapters", who, (long long)MAX_ADAPTERS);
+  // the tile records and the kernels' address set-up keep index positions and pool rows in 32 bits
+  if (pool->a_loc_len > 0x7fffffff || pool->w_rows > 0x7fffffff)
+    return fail(MLORA_ERR_NO_KERNEL, "%s: more than 2^31 - 1 index entries or pool rows", who);
+  return MLORA_OK;
+}
+
+// the plan must have been cut for the pool index it is used with
+int check_plan_pool(const mlora_plan *plan, const mlora_pool *pool, const char *who) {
+  if (plan->n_adapters != pool->n_adapters || plan->n_slots != pool->n_slots)
+    return fail(MLORA_ERR_INVALID, "%s: plan was built for %lld adapters with %d slots, the pool has %lld with %d (a plan "
+                "does not outlive a change of the adapter index)", who, (long long)plan->n_adapters, plan->n_slots,
+                (long long)pool->n_adapters, pool->n_slots);
   return MLORA_OK;
 }
 
@@ -80,31 +92,6 @@ int check_dims(int64_t T, int64_t wide, int64_t narrow, int64_t h_in, int64_t h_
     return fail(MLORA_ERR_NO_KERNEL, "No suitable kernel. h_in=%lld h_out=%lld dtype=%s", (long long)h_in,
                 (long long)h_out, dtype_name(dt));
   return MLORA_OK;
-}
-
-// defaults measured on MI355X (see valora_amd/tile_table.json for the per-shape table the Python
-// host layer uses): 128-token LDS-staged tiles once adapters own long runs of tokens
-int default_bm_shrink(int64_t T, int64_t A) {
-  const int64_t groups = A < T ? (A > 0 ? A : 1) : (T > 0 ? T : 1);
-  if (T > 4096 && T / groups >= 64) return 128;
-  return T <= 1024 ? 16 : 32;
-}
-int default_bm_expand(int64_t T, int64_t A) {
-  (void)A;
-  return T <= 1024 ? 16 : T <= 4096 ? 32 : 128;
-}
-int default_ksplit(int64_t T, int64_t A, int bm, int64_t h_in) {
-  // aim for >= ~1024 workgroups, keep >= 256 K elements per workgroup, at most 16 partials
-  int64_t tiles = tiles_upper(T, A, bm);
-  if (tiles > T) tiles = T;
-  if (tiles < 1) tiles = 1;
-  int64_t ks = (768 + tiles - 1) / tiles;
-  int64_t kmax = h_in / 256;
-  if (kmax < 1) kmax = 1;
-  if (ks > kmax) ks = kmax;
-  if (ks > 16) ks = 16;
-  if (ks < 1) ks = 1;
-  return (int)ks;
 }
 
 }  // namespace
@@ -173,7 +160,7 @@ size_t mlora_one_launch_scratch_bytes(int64_t T, int64_t n_adapters, int64_t max
 size_t mlora_workspace_bytes(int64_t T, int64_t n_adapters, int64_t max_rank) {
   if (T < 0 || n_adapters < 0 || max_rank < 0) return 0;
   auto up = [](size_t n) { return (n + 255) & ~(size_t)255; };
-  const int ks = default_ksplit(T, n_adapters, default_bm_shrink(T, n_adapters), 1 << 16);
+  const int ks = tile_max_ksplit(T, max_rank, n_adapters);
   return up(mlora_plan_bytes(T, n_adapters)) + up(scratch_bytes(T, max_rank, ks)) + up((size_t)T * 8 + 8) + 256;
 }
 
@@ -188,8 +175,11 @@ int mlora_build_plan(void *stream, mlora_plan *plan, const int64_t *ids, int64_t
   if (T > 0 && !ids) return fail(MLORA_ERR_INVALID, "build_plan: ids is null");
   if (n_adapters > 0 && (!a_start || !a_len)) return fail(MLORA_ERR_INVALID, "build_plan: a_start / a_len is null");
   if (n_slots < 1) return fail(MLORA_ERR_INVALID, "build_plan: n_slots must be >= 1");
-  if (bm_shrink == 0) bm_shrink = default_bm_shrink(T, n_adapters);
-  if (bm_expand == 0) bm_expand = default_bm_expand(T, n_adapters);
+  if (bm_shrink == 0 || bm_expand == 0) {   // neither rank nor width is known here: the rule's tile heights
+    const mlora_tile_config c = tile_fallback(T, 16, 4096, n_adapters);
+    if (bm_shrink == 0) bm_shrink = c.bm_shrink;
+    if (bm_expand == 0) bm_expand = c.bm_expand;
+  }
   if (bm_shrink != 16 && bm_shrink != 32 && bm_shrink != 64 && bm_shrink != 128)
     return fail(MLORA_ERR_NO_KERNEL, "build_plan: bm_shrink=%d not in {16,32,64,128}", bm_shrink);
   if (bm_expand < 16 || bm_expand > 256 || (bm_expand % 16) != 0)
@@ -201,6 +191,7 @@ int mlora_build_plan(void *stream, mlora_plan *plan, const int64_t *ids, int64_t
   if (!aligned16(plan->dev)) return fail(MLORA_ERR_INVALID, "build_plan: plan buffer must be 16-byte aligned");
   plan->T = T;
   plan->n_adapters = n_adapters;
+  plan->n_slots = n_slots;
   plan->bm_shrink = bm_shrink;
   plan->bm_expand = bm_expand;
   return launch_plan((hipStream_t)stream, static_cast<int32_t *>(plan->dev), L, ids, a_start, a_len, n_slots,
@@ -243,11 +234,12 @@ int mlora_shrink(void *stream, const mlora_plan *plan, void *scratch, size_t scr
   if (int rc = check_dims(T, h_in, max_rank, h_in, max_rank, dtype)) return rc;
   if (int rc = check_plan(plan, T, "shrink")) return rc;
   if (int rc = check_pool(pool, "shrink")) return rc;
+  if (int rc = check_plan_pool(plan, pool, "shrink")) return rc;
   if (T == 0) return MLORA_OK;
   if (!x || !scratch) return fail(MLORA_ERR_INVALID, "shrink: null pointer");
   if (!aligned16(x) || !aligned16(scratch)) return fail(MLORA_ERR_INVALID, "shrink: x and scratch must be 16-byte aligned");
   if (slot < 0 || slot >= pool->n_slots) return fail(MLORA_ERR_INVALID, "shrink: slot %d outside [0,%d)", slot, pool->n_slots);
-  if (ksplit == 0) ksplit = default_ksplit(T, plan->n_adapters, plan->bm_shrink, h_in);
+  if (ksplit == 0) ksplit = tile_ksplit_for(T, max_rank, h_in, plan->n_adapters, plan->bm_shrink);
   if (ksplit < 1 || ksplit > 64) return fail(MLORA_ERR_INVALID, "shrink: ksplit=%d outside [1,64]", ksplit);
   if (scratch_nbytes < scratch_bytes(T, max_rank, ksplit))
     return fail(MLORA_ERR_WORKSPACE, "shrink: scratch has %zu bytes, needs %zu", scratch_nbytes,
@@ -305,6 +297,7 @@ int mlora_expand(void *stream, const mlora_plan *plan, void *y, int64_t T, int64
   if (int rc = check_dims(T, h_out, max_rank, max_rank, h_out, dtype)) return rc;
   if (int rc = check_plan(plan, T, "expand")) return rc;
   if (int rc = check_pool(pool, "expand")) return rc;
+  if (int rc = check_plan_pool(plan, pool, "expand")) return rc;
   if (T == 0) return MLORA_OK;
   if (!y || !scales) return fail(MLORA_ERR_INVALID, "expand: null pointer");
   if (!scratch && !v) return fail(MLORA_ERR_INVALID, "expand: neither scratch nor v given");
@@ -366,7 +359,7 @@ int mlora_lora_apply(void *stream, const mlora_plan *plan, void *scratch, size_t
     return mlora_lora_apply_multi(stream, plan, scratch, scratch_nbytes, x, T, h_in, h_out, max_rank, pool_a, 1, &tg,
                                   scales, ksplit, flags, dtype);
   }
-  if (ksplit == 0) ksplit = default_ksplit(T, plan->n_adapters, plan->bm_shrink, h_in);
+  if (ksplit == 0) ksplit = tile_ksplit_for(T, max_rank, h_in, plan->n_adapters, plan->bm_shrink);
   if (int rc = mlora_shrink(stream, plan, scratch, scratch_nbytes, x, T, h_in, max_rank, pool_a, slot, ksplit, nullptr,
                             0, MLORA_SHRINK_OVERWRITE, 0, flags, dtype))
     return rc;
@@ -383,6 +376,7 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
   if (int rc = check_dims(T, h_out, max_rank, h_in, h_out, dtype)) return rc;
   if (int rc = check_plan(plan, T, "lora_apply_multi")) return rc;
   if (int rc = check_pool(pool_a, "lora_apply_multi")) return rc;
+  if (int rc = check_plan_pool(plan, pool_a, "lora_apply_multi")) return rc;
   if (n_targets < 1 || n_targets > MLORA_MAX_TARGETS || !targets)
     return fail(MLORA_ERR_INVALID, "lora_apply_multi: n_targets=%d outside [1,%d]", n_targets, MLORA_MAX_TARGETS);
   if (T == 0) return MLORA_OK;
@@ -396,7 +390,7 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
     for (int j = 0; j < i; ++j)
       if (targets[j].y == targets[i].y) return fail(MLORA_ERR_INVALID, "lora_apply_multi: targets %d and %d share y", j, i);
   }
-  if (ksplit == 0) ksplit = default_ksplit(T, plan->n_adapters, plan->bm_shrink, h_in);
+  if (ksplit == 0) ksplit = tile_ksplit_for(T, max_rank, h_in, plan->n_adapters, plan->bm_shrink);
   const bool one_launch = (flags & MLORA_ONE_LAUNCH) != 0;
   if (one_launch) {
     if (plan->bm_shrink != 16 || plan->bm_expand != 16)
@@ -513,9 +507,11 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
 
 // ---- one-call entry points ------------------------------------------------------------------------
 
+// `given`: the caller's plan for exactly these per-token ids (then nothing is built here and the tile heights
+// are the plan's), or null: a plan is built in the workspace with the table's tiles for this shape.
 static int one_call(void *stream, void *y, const void *x, const mlora_pool *pool, const int64_t *ids, int64_t qkvo,
                     const void *scales, int64_t T, int64_t h_in, int64_t h_out, mlora_dtype dtype, int shrink_mode,
-                    int shrink_width, int64_t narrow_stride, Carver &ws, const char *who) {
+                    int shrink_width, int64_t narrow_stride, Carver &ws, const mlora_plan *given, const char *who) {
   if (int rc = check_pool(pool, who)) return rc;
   if (qkvo < 0 || qkvo >= pool->n_slots) return fail(MLORA_ERR_INVALID, "%s: qkvo=%lld outside [0,%d)", who, (long long)qkvo, pool->n_slots);
   const bool expand = h_in < h_out;  // valora/csrc/bgmv/bgmv_impl.cuh:221
@@ -523,58 +519,76 @@ static int one_call(void *stream, void *y, const void *x, const mlora_pool *pool
   const int64_t wide = expand ? h_out : h_in;
   if (int rc = check_dims(T, wide, narrow, h_in, h_out, dtype)) return rc;
   if (T == 0) return MLORA_OK;
-  mlora_plan plan;
-  plan.bytes = mlora_plan_bytes(T, pool->n_adapters);
-  plan.dev = ws.take(plan.bytes);
-  if (!plan.dev) return fail(MLORA_ERR_WORKSPACE, "%s: workspace too small (needs %zu bytes)", who,
-                             mlora_workspace_bytes(T, pool->n_adapters, narrow));
-  if (int rc = mlora_build_plan(stream, &plan, ids, T, pool->a_start, pool->a_len, pool->n_adapters, pool->n_slots, 0, 0))
-    return rc;
+  mlora_plan built;
+  const mlora_plan *plan = given;
+  int ksplit;
+  if (given) {
+    if (int rc = check_plan(given, T, who)) return rc;
+    if (int rc = check_plan_pool(given, pool, who)) return rc;
+    ksplit = tile_ksplit_for(T, narrow, wide, pool->n_adapters, given->bm_shrink);
+  } else {
+    const mlora_tile_config cfg = tile_lookup(T, narrow, wide, pool->n_adapters);
+    built.bytes = mlora_plan_bytes(T, pool->n_adapters);
+    built.dev = ws.take(built.bytes);
+    if (!built.dev) return fail(MLORA_ERR_WORKSPACE, "%s: workspace too small (needs %zu bytes)", who,
+                                mlora_workspace_bytes(T, pool->n_adapters, narrow));
+    if (int rc = mlora_build_plan(stream, &built, ids, T, pool->a_start, pool->a_len, pool->n_adapters, pool->n_slots,
+                                  cfg.bm_shrink, cfg.bm_expand))
+      return rc;
+    plan = &built;
+    ksplit = cfg.ksplit;
+  }
   if (expand) {
     if (narrow_stride == 0) narrow_stride = h_in;
-    return mlora_expand(stream, &plan, y, T, h_out, nullptr, x, narrow_stride, narrow, pool, (int32_t)qkvo, scales, 1,
+    return mlora_expand(stream, plan, y, T, h_out, nullptr, x, narrow_stride, narrow, pool, (int32_t)qkvo, scales, 1,
                         0, dtype);
   }
-  const int ksplit = default_ksplit(T, pool->n_adapters, plan.bm_shrink, h_in);
   const size_t sbytes = scratch_bytes(T, narrow, ksplit);
   void *scratch = ws.take(sbytes);
   if (!scratch) return fail(MLORA_ERR_WORKSPACE, "%s: workspace too small (needs %zu bytes)", who,
                             mlora_workspace_bytes(T, pool->n_adapters, narrow));
   if (narrow_stride == 0) narrow_stride = h_out;
-  return mlora_shrink(stream, &plan, scratch, sbytes, x, T, h_in, narrow, pool, (int32_t)qkvo, ksplit, y,
+  return mlora_shrink(stream, plan, scratch, sbytes, x, T, h_in, narrow, pool, (int32_t)qkvo, ksplit, y,
                       narrow_stride, shrink_mode, shrink_width, 0, dtype);
 }
 
 int mlora_dispatch_bgmv(void *stream, void *y, const void *x, const mlora_pool *pool, const int64_t *indicies,
                         int64_t qkvo, const void *lora_scales, int64_t T, int64_t h_in, int64_t h_out,
-                        mlora_dtype dtype, void *workspace, size_t workspace_bytes) {
+                        mlora_dtype dtype, void *workspace, size_t workspace_bytes, const mlora_plan *plan) {
   if (int rc = check_dtype(dtype, h_in, h_out)) return rc;
-  if (T > 0 && (!y || !x || !indicies)) return fail(MLORA_ERR_INVALID, "dispatch_bgmv: null pointer");
-  if (T > 0 && (!workspace || !aligned16(workspace))) return fail(MLORA_ERR_WORKSPACE, "dispatch_bgmv: workspace missing or misaligned");
+  if (T > 0 && (!y || !x || (!indicies && !plan))) return fail(MLORA_ERR_INVALID, "dispatch_bgmv: null pointer");
+  const bool needs_ws = !(plan && h_in < h_out);   // an expand on a caller-held plan needs no scratch at all
+  if (T > 0 && needs_ws && (!workspace || !aligned16(workspace)))
+    return fail(MLORA_ERR_WORKSPACE, "dispatch_bgmv: workspace missing or misaligned");
   if (T > 0 && h_in < h_out && !lora_scales) return fail(MLORA_ERR_INVALID, "dispatch_bgmv: lora_scales is null");
   Carver ws{static_cast<char *>(workspace), workspace_bytes};
   return one_call(stream, y, x, pool, indicies, qkvo, lora_scales, T, h_in, h_out, dtype, MLORA_SHRINK_OVERWRITE, 0, 0,
-                  ws, "dispatch_bgmv");
+                  ws, plan, "dispatch_bgmv");
 }
 
 int mlora_dispatch_sgmm(void *stream, void *y, const void *x, const mlora_pool *pool, const int64_t *indicies,
                         int64_t qkvo, const void *lora_scales, const int64_t *output_counts,
                         const int64_t *start_ids, int64_t num_problems, int64_t T, int64_t h_in, int64_t h_out,
-                        mlora_dtype dtype, int32_t shrink_mode, void *workspace, size_t workspace_bytes) {
+                        mlora_dtype dtype, int32_t shrink_mode, void *workspace, size_t workspace_bytes,
+                        const mlora_plan *plan) {
   if (int rc = check_dtype(dtype, h_in, h_out)) return rc;
   if (T < 0 || T > MAX_TOKENS) return fail(MLORA_ERR_INVALID, "dispatch_sgmm: T=%lld out of range", (long long)T);
   if (num_problems < 0) return fail(MLORA_ERR_INVALID, "dispatch_sgmm: num_problems < 0");
   if (shrink_mode != MLORA_SHRINK_OVERWRITE && shrink_mode != MLORA_SHRINK_ACCUMULATE)
     return fail(MLORA_ERR_INVALID, "dispatch_sgmm: bad shrink_mode %d", shrink_mode);
   if (T == 0) return MLORA_OK;
-  if (!y || !x || !indicies) return fail(MLORA_ERR_INVALID, "dispatch_sgmm: null pointer");
-  if (!workspace || !aligned16(workspace)) return fail(MLORA_ERR_WORKSPACE, "dispatch_sgmm: workspace missing or misaligned");
+  if (!y || !x || (!indicies && !plan)) return fail(MLORA_ERR_INVALID, "dispatch_sgmm: null pointer");
+  if (!(plan && (h_in < h_out)) && (!workspace || !aligned16(workspace)))
+    return fail(MLORA_ERR_WORKSPACE, "dispatch_sgmm: workspace missing or misaligned");
   if (h_in < h_out && !lora_scales) return fail(MLORA_ERR_INVALID, "dispatch_sgmm: lora_scales is null");
   Carver ws{static_cast<char *>(workspace), workspace_bytes};
-  int64_t *ids_eff = static_cast<int64_t *>(ws.take((size_t)T * 8));
-  if (!ids_eff) return fail(MLORA_ERR_WORKSPACE, "dispatch_sgmm: workspace too small");
-  if (int rc = mlora_ids_from_segments(stream, ids_eff, indicies, start_ids, output_counts, num_problems, T)) return rc;
-  return one_call(stream, y, x, pool, ids_eff, qkvo, lora_scales, T, h_in, h_out, dtype, shrink_mode, 0, 0, ws,
+  int64_t *ids_eff = nullptr;
+  if (!plan) {   // a caller-held plan was cut from the covered rows' ids already
+    ids_eff = static_cast<int64_t *>(ws.take((size_t)T * 8));
+    if (!ids_eff) return fail(MLORA_ERR_WORKSPACE, "dispatch_sgmm: workspace too small");
+    if (int rc = mlora_ids_from_segments(stream, ids_eff, indicies, start_ids, output_counts, num_problems, T)) return rc;
+  }
+  return one_call(stream, y, x, pool, ids_eff, qkvo, lora_scales, T, h_in, h_out, dtype, shrink_mode, 0, 0, ws, plan,
                   "dispatch_sgmm");
 }
 
@@ -627,53 +641,61 @@ int mlora_dispatch_bgmv_static(void *stream, void *y, const void *x, const mlora
   // kernels read, and every split-K partial is written before it is summed
   Carver ws{static_cast<char *>(ws_dev), STATIC_WS_BYTES};
   return one_call(stream, y, x, pool, indicies, qkvo, lora_scales, T, h_in, h_out, dtype, MLORA_SHRINK_OVERWRITE, 0, 0,
-                  ws, "dispatch_bgmv_static");
+                  ws, nullptr, "dispatch_bgmv_static");
 }
 
 int mlora_prefill_shrink(void *stream, void *o, const void *x, const mlora_pool *pool, const int32_t *b_start_loc,
                          const int32_t *b_seq_len, const int64_t *b_indicies, int64_t n_req, int64_t T,
                          int64_t hidden, int64_t o_stride, int64_t qkvo, int64_t max_rank, int64_t max_input_len,
-                         mlora_dtype dtype, void *workspace, size_t workspace_bytes) {
+                         mlora_dtype dtype, void *workspace, size_t workspace_bytes, const mlora_plan *plan) {
   if (int rc = check_dtype(dtype, hidden, max_rank)) return rc;
   if (T < 0 || T > MAX_TOKENS || n_req < 0) return fail(MLORA_ERR_INVALID, "prefill_shrink: bad size");
   if (T == 0 || n_req == 0) return MLORA_OK;
   if (!o || !x) return fail(MLORA_ERR_INVALID, "prefill_shrink: null pointer");
-  if (!workspace || !aligned16(workspace)) return fail(MLORA_ERR_WORKSPACE, "prefill_shrink: workspace missing or misaligned");
+  if (!(plan && (false)) && (!workspace || !aligned16(workspace)))
+    return fail(MLORA_ERR_WORKSPACE, "prefill_shrink: workspace missing or misaligned");
   if (max_rank <= 0 || max_rank > MAX_RANK) return fail(MLORA_ERR_NO_KERNEL, "prefill_shrink: max_rank=%lld", (long long)max_rank);
   Carver ws{static_cast<char *>(workspace), workspace_bytes};
-  int64_t *ids_eff = static_cast<int64_t *>(ws.take((size_t)T * 8));
-  if (!ids_eff) return fail(MLORA_ERR_WORKSPACE, "prefill_shrink: workspace too small");
-  // rows visited per request: grid z covers cdiv(max_input_len, 32) blocks of 32 rows (lora_prefill.py:147)
-  const int64_t max_rows = (max_input_len + 31) / 32 * 32;
-  if (int rc = mlora_ids_from_requests(stream, ids_eff, b_start_loc, b_seq_len, b_indicies, n_req, T, max_rows)) return rc;
+  int64_t *ids_eff = nullptr;
+  if (!plan) {
+    ids_eff = static_cast<int64_t *>(ws.take((size_t)T * 8));
+    if (!ids_eff) return fail(MLORA_ERR_WORKSPACE, "prefill_shrink: workspace too small");
+    // rows visited per request: grid z covers cdiv(max_input_len, 32) blocks of 32 rows (lora_prefill.py:147)
+    const int64_t max_rows = (max_input_len + 31) / 32 * 32;
+    if (int rc = mlora_ids_from_requests(stream, ids_eff, b_start_loc, b_seq_len, b_indicies, n_req, T, max_rows)) return rc;
+  }
   // columns stored: cdiv(max_rank, BLOCK_N) blocks of BLOCK_N = 16 (or max_rank when <= 8) (lora_prefill.py:142,147)
   const int64_t block_n = max_rank > 8 ? 16 : max_rank;
   int64_t width = (max_rank + block_n - 1) / block_n * block_n;
   if (width > o_stride) width = o_stride;
   const int64_t narrow = align_up(max_rank, 8);
   return one_call(stream, o, x, pool, ids_eff, qkvo, nullptr, T, hidden, narrow, dtype, MLORA_SHRINK_ZERO_PAD,
-                  (int)width, o_stride, ws, "prefill_shrink");
+                  (int)width, o_stride, ws, plan, "prefill_shrink");
 }
 
 int mlora_prefill_expand(void *stream, void *o, const void *x, const mlora_pool *pool, const void *scale,
                          const int32_t *b_start_loc, const int32_t *b_seq_len, const int64_t *b_indicies,
                          int64_t n_req, int64_t T, int64_t x_stride, int64_t feat_out, int64_t qkvo,
                          int64_t max_rank, int64_t max_input_len, mlora_dtype dtype, void *workspace,
-                         size_t workspace_bytes) {
+                         size_t workspace_bytes, const mlora_plan *plan) {
   if (int rc = check_dtype(dtype, max_rank, feat_out)) return rc;
   if (T < 0 || T > MAX_TOKENS || n_req < 0) return fail(MLORA_ERR_INVALID, "prefill_expand: bad size");
   if (T == 0 || n_req == 0) return MLORA_OK;
   if (!o || !x || !scale) return fail(MLORA_ERR_INVALID, "prefill_expand: null pointer");
-  if (!workspace || !aligned16(workspace)) return fail(MLORA_ERR_WORKSPACE, "prefill_expand: workspace missing or misaligned");
+  if (!(plan && (true)) && (!workspace || !aligned16(workspace)))
+    return fail(MLORA_ERR_WORKSPACE, "prefill_expand: workspace missing or misaligned");
   if (max_rank <= 0 || max_rank > MAX_RANK || max_rank >= feat_out)
     return fail(MLORA_ERR_NO_KERNEL, "prefill_expand: max_rank=%lld", (long long)max_rank);
   Carver ws{static_cast<char *>(workspace), workspace_bytes};
-  int64_t *ids_eff = static_cast<int64_t *>(ws.take((size_t)T * 8));
-  if (!ids_eff) return fail(MLORA_ERR_WORKSPACE, "prefill_expand: workspace too small");
-  const int64_t max_rows = (max_input_len + 31) / 32 * 32;
-  if (int rc = mlora_ids_from_requests(stream, ids_eff, b_start_loc, b_seq_len, b_indicies, n_req, T, max_rows)) return rc;
+  int64_t *ids_eff = nullptr;
+  if (!plan) {
+    ids_eff = static_cast<int64_t *>(ws.take((size_t)T * 8));
+    if (!ids_eff) return fail(MLORA_ERR_WORKSPACE, "prefill_expand: workspace too small");
+    const int64_t max_rows = (max_input_len + 31) / 32 * 32;
+    if (int rc = mlora_ids_from_requests(stream, ids_eff, b_start_loc, b_seq_len, b_indicies, n_req, T, max_rows)) return rc;
+  }
   return one_call(stream, o, x, pool, ids_eff, qkvo, scale, T, align_up(max_rank, 8), feat_out, dtype,
-                  MLORA_SHRINK_OVERWRITE, 0, x_stride, ws, "prefill_expand");
+                  MLORA_SHRINK_OVERWRITE, 0, x_stride, ws, plan, "prefill_expand");
 }
 
 }  // extern "C"

@@ -67,6 +67,12 @@ static inline int64_t partial_stride(int64_t max_rank) { return align_up(max_ran
 int fail(int code, const char *fmt, ...);
 int check_launch(const char *what);
 
+// ---- tile table (tiles.hip) --------------------------------------------------------------------
+mlora_tile_config tile_lookup(int64_t T, int64_t max_rank, int64_t hidden, int64_t A);
+mlora_tile_config tile_fallback(int64_t T, int64_t max_rank, int64_t hidden, int64_t A);
+int tile_ksplit_for(int64_t T, int64_t max_rank, int64_t hidden, int64_t A, int bm);
+int tile_max_ksplit(int64_t T, int64_t max_rank, int64_t A);
+
 // ---- kernel launchers ------------------------------------------------------------------------
 struct PoolDev {
   const uint16_t *w;

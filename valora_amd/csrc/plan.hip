@@ -207,13 +207,14 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
       const int k = i - toff[a];
       const int c = cnt[a];
       const int64_t st = start_of(a);
-      if (st < 0 || st > 0x7fffffff) atomicOr(&s_err, (int)PERR_START_OVERFLOW);
+      const bool st_bad = st < 0 || st > 0x7fffffff;
+      if (st_bad) atomicOr(&s_err, (int)PERR_START_OVERFLOW);
       int32_t *tl = tiles + (int64_t)i * TILE_WORDS;
       tl[0] = a;
       tl[1] = rank_of(a);
       tl[2] = gstart[a] + k * bm;
       tl[3] = min(bm, c - k * bm);
-      tl[4] = (int32_t)st;
+      tl[4] = st_bad ? INT32_MIN / 2 : (int32_t)st;   // an index position no look-up accepts
       tl[5] = 0; tl[6] = 0; tl[7] = 0;
     }
     // the kernels' grids are sized with the upper bound of the tile count: records past the last

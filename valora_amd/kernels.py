@@ -83,7 +83,7 @@ def dispatch_bgmv(y, x, w, start_indicies, lora_ranks, loc_indicies, indicies, q
     ws = _workspace(T, start_indicies.numel(), narrow, x.device)
     _lib.check(_lib.lib().mlora_dispatch_bgmv(
         stream, _lib.ptr(y), _lib.ptr(x), pool, _lib.ptr(indicies), int(qkvo),
-        _lib.ptr(lora_scales), T, h_in, h_out, code, _lib.ptr(ws), ws.numel()))
+        _lib.ptr(lora_scales), T, h_in, h_out, code, _lib.ptr(ws), ws.numel(), None))
 
 
 def _planned_call(plan, stream, y, x, pool, qkvo, scales, T, h_in, h_out, code, shrink_mode=_lib.SHRINK_OVERWRITE,
@@ -117,8 +117,5 @@ def _cached_plan(ids, a_start, a_len, T, narrow, wide, n_slots=4, extra_tensors=
         plan.ids_keepalive = eff
         return plan
 
-    try:
-        return _plan_cache.lookup((ids, a_start, a_len) + tuple(extra_tensors),
-                                  (T, narrow, wide, n_slots, ids.device.index) + tuple(extra_scalars), build)
-    except RuntimeError:
-        return None
+    return _plan_cache.lookup((ids, a_start, a_len) + tuple(extra_tensors),
+                              (T, narrow, wide, n_slots, ids.device.index) + tuple(extra_scalars), build)

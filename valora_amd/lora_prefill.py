@@ -63,7 +63,7 @@ def lora_get_qkvo_fwd_shrink(x, w, o, b_loc, b_lora_start, b_lora_ranks, b_start
     _lib.check(_lib.lib().mlora_prefill_shrink(
         _lib.current_stream(x.device), _lib.ptr(o), _lib.ptr(x), pool, _lib.ptr(s), _lib.ptr(n),
         _lib.ptr(idx), n.numel(), T, int(hidden_size), o.stride(0), int(qkvo), int(max_rank),
-        int(max_input_len), code, _lib.ptr(ws), ws.numel()))
+        int(max_input_len), code, _lib.ptr(ws), ws.numel(), None))
 
 
 @torch.inference_mode()
@@ -91,4 +91,4 @@ def lora_get_qkvo_fwd_expand(x, w, o, scale, b_loc, b_lora_start, b_lora_ranks, 
     _lib.check(_lib.lib().mlora_prefill_expand(
         _lib.current_stream(x.device), _lib.ptr(o), _lib.ptr(x), pool, _lib.ptr(scale), _lib.ptr(s),
         _lib.ptr(n), _lib.ptr(idx), n.numel(), T, x.stride(0), int(feat_out), int(qkvo), int(max_rank),
-        int(max_input_len), code, _lib.ptr(ws), ws.numel()))
+        int(max_input_len), code, _lib.ptr(ws), ws.numel(), None))

@@ -8,15 +8,13 @@ fall back to a fixed shape for unknown keys.  Here the key is
 vary: the token height of a shrink tile, the split-K factor of the shrink, who sums the split-K
 chunks and the token height of an expand tile.  Entries come from sweeps on MI355X (``tile_table.json`` next to this file);
 a width without entries uses those of the nearest measured width, and anything else falls back to a
-rule, like the reference's fallback tuple.
+rule, like the reference's fallback tuple.  The look-up itself lives in the library
+(``csrc/tiles.hip``, table generated from the JSON file at build time); this module is its Python face.
 """
 from __future__ import annotations
 
-import json
-import math
 import os
 from dataclasses import dataclass
-from typing import Dict
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 TABLE_PATH = os.path.join(_HERE, "tile_table.json")
@@ -47,50 +45,26 @@ def key(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> str:
             f"{_bucket(n_adapters, ADAPTER_BUCKETS)}")
 
 
+def _cfg(c) -> TileConfig:
+    from . import _lib
+    return TileConfig(int(c.bm_shrink), int(c.ksplit), int(c.bm_expand), bool(c.flags & _lib.REDUCE_IN_EXPAND),
+                      bool(c.flags & _lib.ONE_LAUNCH))
+
+
 def fallback(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> TileConfig:
-    tokens_per_adapter = n_tokens / max(1, min(n_adapters, n_tokens))
-    if n_tokens > 4096 and tokens_per_adapter >= 64:
-        bm_s = 128
-    else:
-        bm_s = 16 if n_tokens <= 1024 else 32
-    tiles = max(1, min(n_tokens, -(-n_tokens // bm_s) + min(n_adapters, n_tokens)))
-    ksplit = max(1, min(16, hidden // 256, -(-768 // tiles)))
-    bm_e = 16 if n_tokens <= 1024 else 32 if n_tokens <= 4096 else 128
-    return TileConfig(bm_s, ksplit, bm_e, n_tokens <= 1024)
-
-
-_table: Dict[str, TileConfig] = {}
-_hiddens: list = []      # the widths the table has entries for
-_loaded = False
-
-
-def _load() -> None:
-    global _loaded
-    _loaded = True
-    if os.path.exists(TABLE_PATH):
-        with open(TABLE_PATH) as f:
-            raw = json.load(f)
-        for k, v in raw.get("entries", {}).items():
-            _table[k] = TileConfig(int(v["bm_shrink"]), int(v["ksplit"]), int(v["bm_expand"]),
-                                   bool(v.get("reduce_in_expand", False)), bool(v.get("one_launch", False)))
-        _hiddens[:] = sorted({int(k.split(":")[2]) for k in _table})
+    """The rule a shape without a table entry gets (``mlora_tile_fallback``)."""
+    from . import _lib
+    c = _lib.TileConfig()
+    _lib.check(_lib.lib().mlora_tile_fallback(int(n_tokens), int(max_rank), int(hidden), int(n_adapters), c))
+    return _cfg(c)
 
 
 def lookup(n_tokens: int, max_rank: int, hidden: int, n_adapters: int) -> TileConfig:
-    if not _loaded:
-        _load()
-    cfg = _table.get(key(n_tokens, max_rank, hidden, n_adapters))
-    if cfg is None and _hiddens:
-        # a width the table was not measured for: the entry of the nearest measured width (ratio-wise),
-        # with the split-K factor cut to what the width can be split into
-        near = min(_hiddens, key=lambda h: abs(math.log(h / max(1, hidden))))
-        cfg = _table.get(key(n_tokens, max_rank, near, n_adapters))
-        if cfg is not None:
-            cfg = TileConfig(cfg.bm_shrink, max(1, min(cfg.ksplit, hidden // 128)), cfg.bm_expand,
-                             cfg.reduce_in_expand and min(cfg.ksplit, hidden // 128) > 1,
-                             cfg.one_launch and hidden >= 256)
-    if cfg is None:
-        return fallback(n_tokens, max_rank, hidden, n_adapters)
-    if max_rank > 64 and cfg.bm_shrink == 64:     # ranks above 64 have no 64-token shrink tile
-        cfg = TileConfig(32, cfg.ksplit, cfg.bm_expand, cfg.reduce_in_expand, False)
-    return cfg
+    """The configuration ``libmlora.so`` itself uses for this shape (``mlora_tile_lookup``): the table is
+    compiled into the library, so the Python host layer and any other caller of the C ABI agree.  After
+    ``tune_tiles`` has rewritten ``tile_table.json`` the library has to be rebuilt
+    (``python -m valora_amd._build``) for new entries to take effect."""
+    from . import _lib
+    c = _lib.TileConfig()
+    _lib.check(_lib.lib().mlora_tile_lookup(int(n_tokens), int(max_rank), int(hidden), int(n_adapters), c))
+    return _cfg(c)
