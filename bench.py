@@ -38,6 +38,8 @@ def parse():
     ap.add_argument("--layers", type=int, default=32)
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly from Python instead of replaying a HIP graph")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the layer, drop-in entry point and step legs")
+    ap.add_argument("--no-step5", action="store_true", help="skip the 32-layer serving step of configuration 5")
     ap.add_argument("--bm-shrink", type=int, default=None)
     ap.add_argument("--bm-expand", type=int, default=None)
     ap.add_argument("--ksplit", type=int, default=None)
@@ -426,6 +428,84 @@ def bench_adapter_residency(torch, dev):
     return out
 
 
+def bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, reps, no_step5):
+    """Legs beside the headline, all on the config-2 decode shape with the same rotation over `L` layers'
+    buffers: a whole attention block's LoRA work per layer, and the same shrink + expand pair reached through
+    each of the reference's entry points (what an unchanged caller of the reference gets), replayed from a HIP
+    graph and launched eagerly from Python."""
+    from valora_amd import atmm_ops, kernels, lora_prefill
+    p = wd.targets[0].pool
+    idx = (p.a_start, p.a_len, p.a_loc)
+    T, H, R = w.T, 4096, 16
+    ids = wd.ids
+    g = torch.Generator(device=dev).manual_seed(2003)
+    rnd = lambda: torch.randn(T, H, generator=g, device=dev).to(w.dtype)
+    out = {}
+
+    # -- one layer's attention LoRA: q, k, v read the same x (one call), o reads the attention output
+    plan = LoraPlan(ids, p.a_start, p.a_len, R, hidden=H)
+    yk, yv, yo = [rnd() for _ in range(L)], [rnd() for _ in range(L)], [rnd() for _ in range(L)]
+
+    def layer():
+        for l in range(L):
+            plan.apply_multi([ys[l], yk[l], yv[l]], xs[l], kb[l], vb[l], *idx, (0, 1, 2), p.a_scaling)
+            plan.apply(yo[l], xs[(l + 1) % L], kb[l], vb[l], *idx, 3, p.a_scaling)
+
+    ms, _ = time_graph(torch, layer, reps, 5, use_graph)
+    out["layer_us"] = round(ms * 1e3 / L, 3)
+    out["layer_us_is"] = "q+k+v in one mlora_lora_apply_multi call + o in one mlora_lora_apply call, per layer"
+    del yk, yv, yo
+
+    # -- the reference's entry points: delta = shrink(x); y += expand(delta), two calls per layer
+    delta = [torch.zeros(T, R, dtype=w.dtype, device=dev) for _ in range(L)]
+
+    def bgmv_pair():
+        for l in range(L):
+            kernels.dispatch_bgmv(delta[l], xs[l], kb[l], *idx, ids, 0, p.a_scaling)
+            kernels.dispatch_bgmv(ys[l], delta[l], vb[l], *idx, ids, 0, p.a_scaling)
+
+    from valora_amd import segments
+    oc, rc, li, st, n_runs = segments.count_consecutive_requests(p.a_len, ids)   # runs of equal ids, as the
+    P = int(n_runs.item())                                                        # reference's caller builds them
+    tmp = torch.empty(256, dtype=torch.uint8, device=dev)
+
+    def sgmm_pair():
+        for l in range(L):
+            atmm_ops.dispatch_bgmv(delta[l], xs[l], kb[l], *idx, ids, 0, p.a_scaling, oc, rc, li, st, tmp, P,
+                                   64, 32, 32, 32, 32, 32)
+            atmm_ops.dispatch_bgmv(ys[l], delta[l], vb[l], *idx, ids, 0, p.a_scaling, oc, rc, li, st, tmp, P,
+                                   32, 64, 32, 32, 32, 32)
+
+    b_start = torch.arange(T, dtype=torch.int32, device=dev)
+    b_len = torch.ones(T, dtype=torch.int32, device=dev)
+
+    def prefill_pair():
+        for l in range(L):
+            lora_prefill.lora_get_qkvo_fwd_shrink(xs[l], kb[l], delta[l], p.a_loc, p.a_start, p.a_len, b_start, b_len,
+                                                  ids, H, 0, R, 1)
+            lora_prefill.lora_get_qkvo_fwd_expand(delta[l], vb[l], ys[l], p.a_scaling, p.a_loc, p.a_start, p.a_len,
+                                                  b_start, b_len, ids, H, 0, R, 1)
+
+    legs = {}
+    for name, fn in (("valora._kernels.dispatch_bgmv", bgmv_pair), ("atmm_ops.dispatch_bgmv", sgmm_pair),
+                     ("lora_prefill.lora_get_qkvo_fwd_*", prefill_pair)):
+        ev_g, _ = time_graph(torch, fn, reps, 5, True)
+        ev_e, wall_e = time_graph(torch, fn, max(10, reps // 4), 3, False)
+        legs[name] = {"graph_us_per_layer": round(ev_g * 1e3 / L, 3), "eager_us_per_layer": round(ev_e * 1e3 / L, 3),
+                      "eager_host_us_per_layer": round(wall_e * 1e3 / L, 3)}
+    out["dropin_pair"] = legs
+    out["dropin_pair_is"] = ("shrink + expand of the config-2 op through the reference's own entry points (two calls per "
+                             "layer, torch binding -> one C-ABI call each with the cached plan of the batch); graph = HIP "
+                             "graph replay, eager = launched from Python call by call (events / host wall clock)")
+    if not no_step5:
+        try:
+            s5 = bench_config5_step(torch, W, dev, use_graph)
+            out["config5_step"] = s5
+        except Exception as exc:    # the headline does not depend on this leg
+            out["config5_step"] = {"error": f"{type(exc).__name__}: {exc}"}
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -460,9 +540,15 @@ def main():
 
     fused = plan.one_launch
 
-    def step():
+    def layers_only():
         for l in range(L):
             plan.apply(ys[l], xs[l], kb[l], vb[l], *idx, 0, p.a_scaling)
+
+    def step():
+        # what a serving step does for this op: sort the batch's tokens by adapter and cut the tiles ONCE
+        # (the reference rebuilds its segment tensors once per forward, model_rpc.py:381), then one op per layer
+        plan.rebuild()
+        layers_only()
 
     def shrink_only():
         for l in range(L):
@@ -499,7 +585,8 @@ def main():
     reps = max(10, min(args.steps, 200))
     sh_ms, _ = time_graph(torch, shrink_only, reps, 5, use_graph)
     ex_ms, _ = time_graph(torch, expand_only, reps, 5, use_graph)
-    op_ms, _ = time_graph(torch, step, reps, 5, use_graph)
+    op_ms, _ = time_graph(torch, layers_only, reps, 5, use_graph)
+    plan_ms, _ = time_graph(torch, plan.rebuild, reps, 5, use_graph)
     sh_us, ex_us, op_us = sh_ms * 1e3 / L, ex_ms * 1e3 / L, op_ms * 1e3 / L
 
     s_el = 2
@@ -520,7 +607,8 @@ def main():
                 "shrink_kernel_us": round(sh_us, 3), "expand_kernel_us": round(ex_us, 3),
                 "op_bytes": bytes_op, "op_us_events": round(op_us, 3),
                 "op_achieved_gbps": round(bytes_op / (op_us * 1e-6) / 1e9, 1),
-                "method": "HIP events on the launch stream around %d graph replays of %d launches" % (reps, L)}
+                "method": "HIP events on the launch stream around %d graph replays of %d launches (the op alone, "
+                          "without the once-per-step plan build)" % (reps, L)}
 
     out = {
         "metric": "lora_op_us_per_layer", "value": round(us_per_layer, 3), "unit": "us/layer", "n_gpus": 1,
@@ -528,6 +616,8 @@ def main():
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "config2 decode BGMV: 256 tokens (1/request), 64 adapters rank 16, Zipf(0.6) ids, "
                                "4096->4096, fp16, shrink+expand; one step = this op on %d layers" % L,
+                   "step": "mlora_build_plan (token sort + tile cut, once per step) + the op on every layer, all "
+                           "inside the timed region" + (", one hip graph" if use_graph else ""),
                    "layers_per_step": L, "tokens": w.T, "adapters_touched": len(used),
                    "launch": "hip graph replay" if use_graph else "eager python launches",
                    "kernels": "shrink and expand items of one grid, one launch" if fused else "shrink then expand, two launches",
@@ -535,7 +625,10 @@ def main():
         "hbm_gbps": round(bytes_op / (us_per_layer * 1e-6) / 1e9, 1),
         "hbm_frac": round(bytes_op / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
         "roofline": roofline,
+        "plan_us": round(plan_ms * 1e3, 3),
     }
+    if not args.no_extras:
+        out["extra"] = bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, reps, args.no_step5)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(torch, w)
     if args.all_configs:

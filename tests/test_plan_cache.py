@@ -1,6 +1,7 @@
 """Host logic of the plan reuse in the drop-in shims: an entry is reused for tensors that live at the same
 address and have not been modified through PyTorch since -- fresh views of the same memory included -- and
-for the same scalars.  CPU only (the cache holds whatever the builder returns)."""
+for the same scalars.  CPU only: the cache of the compiled binding, driven through its Python face (it holds
+whatever the builder returns)."""
 import torch
 
 from valora_amd import _plan_cache as C
@@ -66,11 +67,11 @@ def test_recycled_addresses_cannot_match():
     seen = set()
     for i in range(50):
         t = torch.full((16,), i, dtype=torch.long)       # a new tensor per 'forward pass', freed by the caller
-        assert t.data_ptr() not in seen or len(C._entries) >= C._MAX_ENTRIES
+        assert t.data_ptr() not in seen or C.size() >= C.max_entries()
         C.lookup((t,), (16,), build)
         seen.add(t.data_ptr())
         del t
-    assert len(built) == 50 and len(C._entries) == C._MAX_ENTRIES
+    assert len(built) == 50 and C.size() == C.max_entries()
 
 
 def test_entries_are_bounded_and_lru():
@@ -86,11 +87,11 @@ def test_entries_are_bounded_and_lru():
         t = torch.zeros(4, dtype=torch.long)
         keep.append(t)
         C.lookup((t,), (i,), build)
-    assert len(C._entries) == C._MAX_ENTRIES
+    assert C.size() == C.max_entries()
     assert C.lookup((keep[-1],), (19,), build) == 20 and n[0] == 20      # the most recent ones are still there
     assert C.lookup((keep[0],), (0,), build) == 21                       # the oldest was evicted and is rebuilt
     C.clear()
-    assert C._entries == []
+    assert C.size() == 0
 
 
 def test_inference_tensors():
@@ -102,18 +103,18 @@ def test_inference_tensors():
         ids = torch.arange(8)
         a = C.lookup((ids,), (8,), build)
         assert C.lookup((ids,), (8,), build) is a and len(built) == 1
-        C.cache_inference_tensors = False
+        C.set_cache_inference_tensors(False)
         try:
             assert C.lookup((ids,), (8,), build) is None and len(built) == 1
         finally:
-            C.cache_inference_tensors = True
+            C.set_cache_inference_tensors(True)
 
 
 def test_disabled_cache_keeps_nothing():
     C.clear()
     C.set_enabled(False)
     try:
-        assert not C.enabled() and C._entries == []
+        assert not C.enabled() and C.size() == 0
     finally:
         C.set_enabled(True)
     assert C.enabled()

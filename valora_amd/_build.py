@@ -1,8 +1,10 @@
-"""Build recipe of ``libmlora.so`` (the HIP kernels + C ABI) for gfx950.
+"""Build recipe of ``libmlora.so`` (the HIP kernels + C ABI) for gfx950, and of the torch binding
+above it.
 
 ``hipcc`` cross-compiles without a GPU, so this runs anywhere the ROCm toolchain is installed.
 The library is built in-tree (``valora_amd/libmlora.so``) and links only against the HIP
-runtime -- no torch, no pybind.
+runtime -- no torch, no pybind.  ``valora_amd/_binding.so`` is host code only (``g++``): the
+reference's op entry points as a torch extension module that calls the library through its C ABI.
 """
 from __future__ import annotations
 
@@ -18,6 +20,8 @@ SOURCES = ["api.hip", "tiles.hip", "plan.hip", "shrink.hip", "expand.hip", "deco
 TABLE_JSON = os.path.join(HERE, "tile_table.json")
 TABLE_INC = os.path.join(CSRC, "tile_table_gen.inc")
 LIB_PATH = os.path.join(HERE, "libmlora.so")
+BINDING_SRC = os.path.join(CSRC, "binding.cpp")
+BINDING_PATH = os.path.join(HERE, "_binding.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -60,16 +64,42 @@ def generate_tile_table() -> str:
     return TABLE_INC
 
 
-def build(verbose: bool = False) -> str:
-    generate_tile_table()
-    cmd = command()
+def binding_command() -> List[str]:
+    """``g++`` line of the torch binding: torch's and Python's headers, HIP's runtime API header (for the
+    stream type), linked against libmlora.so beside it and the torch libraries the process has loaded."""
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        raise RuntimeError("g++ not found: it is required to build the torch binding")
+    inc = cpp_extension.include_paths() + [sysconfig.get_paths()["include"], "/opt/rocm/include",
+                                           os.path.join(ROOT, "include")]
+    libdirs = cpp_extension.library_paths()
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    return ([cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
+             "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_binding",
+             f"-D_GLIBCXX_USE_CXX11_ABI={abi}"] +
+            [a for d in inc for a in ("-isystem", d)] + [BINDING_SRC] +
+            [f"-L{d}" for d in libdirs] + [f"-L{HERE}", "-lmlora", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch",
+                                           "-ltorch_python", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,$ORIGIN"] +
+            [f"-Wl,-rpath,{d}" for d in libdirs] + ["-Wl,-rpath,/opt/rocm/lib", "-o", BINDING_PATH])
+
+
+def _run(cmd: List[str], what: str, verbose: bool) -> None:
     proc = subprocess.run(cmd, capture_output=True, text=True)
-    # the host pass warns that it does not know the packed-fp32 feature; that is expected
+    # hipcc's host pass warns that it does not know the packed-fp32 feature; that is expected
     err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)
     if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + " ".join(cmd) + "\n" + err)
+        raise RuntimeError(f"{what} failed:\n" + " ".join(cmd) + "\n" + err)
     if verbose and err.strip():
         print(err)
+
+
+def build(verbose: bool = False) -> str:
+    generate_tile_table()
+    _run(command(), "hipcc", verbose)
+    _run(binding_command(), "g++ (torch binding)", verbose)
     return LIB_PATH
 
 

@@ -652,7 +652,7 @@ int mlora_prefill_shrink(void *stream, void *o, const void *x, const mlora_pool 
   if (T < 0 || T > MAX_TOKENS || n_req < 0) return fail(MLORA_ERR_INVALID, "prefill_shrink: bad size");
   if (T == 0 || n_req == 0) return MLORA_OK;
   if (!o || !x) return fail(MLORA_ERR_INVALID, "prefill_shrink: null pointer");
-  if (!(plan && (false)) && (!workspace || !aligned16(workspace)))
+  if (!workspace || !aligned16(workspace))
     return fail(MLORA_ERR_WORKSPACE, "prefill_shrink: workspace missing or misaligned");
   if (max_rank <= 0 || max_rank > MAX_RANK) return fail(MLORA_ERR_NO_KERNEL, "prefill_shrink: max_rank=%lld", (long long)max_rank);
   Carver ws{static_cast<char *>(workspace), workspace_bytes};
@@ -682,7 +682,7 @@ int mlora_prefill_expand(void *stream, void *o, const void *x, const mlora_pool 
   if (T < 0 || T > MAX_TOKENS || n_req < 0) return fail(MLORA_ERR_INVALID, "prefill_expand: bad size");
   if (T == 0 || n_req == 0) return MLORA_OK;
   if (!o || !x || !scale) return fail(MLORA_ERR_INVALID, "prefill_expand: null pointer");
-  if (!(plan && (true)) && (!workspace || !aligned16(workspace)))
+  if (!plan && (!workspace || !aligned16(workspace)))
     return fail(MLORA_ERR_WORKSPACE, "prefill_expand: workspace missing or misaligned");
   if (max_rank <= 0 || max_rank > MAX_RANK || max_rank >= feat_out)
     return fail(MLORA_ERR_NO_KERNEL, "prefill_expand: max_rank=%lld", (long long)max_rank);

@@ -176,7 +176,6 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(DecodeArgs a) {
   const int h_out = a.e.h_out;
 
   const int lrow = lane & 15, kg = lane >> 4;
-  const int64_t base = (int64_t)astart + (int64_t)r * slot;
   int o_wave[DEC_CH];
 #pragma unroll
   for (int c = 0; c < DEC_CH; ++c) o_wave[c] = oc * DEC_BN + c * 256 + wave * DEC_WN;

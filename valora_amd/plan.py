@@ -58,10 +58,8 @@ class LoraPlan:
         nbytes = int(L.mlora_plan_bytes(self.T, self.n_adapters))
         self.buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
         self.handle = _lib.Plan(_lib.ptr(self.buf), self.buf.numel(), 0, 0, 0, 0)
-        self._keep = (ids, a_start, a_len)
-        _lib.check(L.mlora_build_plan(_lib.current_stream(self.device), self.handle, _lib.ptr(ids.contiguous()),
-                                      self.T, _lib.ptr(a_start), _lib.ptr(a_len), self.n_adapters, n_slots,
-                                      self.bm_shrink, self.bm_expand))
+        self._keep = (ids.contiguous(), a_start, a_len)
+        self.rebuild()
         # room for a multi-target call from the start: the buffer is never replaced, so a HIP graph captured
         # from this plan or work still queued on another stream keeps pointing at live memory
         self.scratch_per_target = int(L.mlora_scratch_bytes(self.T, self.max_rank, self.ksplit))
@@ -70,6 +68,21 @@ class LoraPlan:
             nbytes = max(nbytes, max(int(L.mlora_one_launch_scratch_bytes(self.T, self.n_adapters, self.max_rank,
                                                                           self.ksplit, n)) for n in (1, 2, 3, 4)))
         self.scratch = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+
+    def rebuild(self, ids: Optional[torch.Tensor] = None) -> None:
+        """Cut the tiles again, in place, for the next batch of the same size (``ids`` of the same length; None
+        re-reads the tensor the plan was made from, whose contents may have changed).  One launch on the current
+        stream, no allocation: a serving loop that replays one HIP graph per step captures this call at the
+        head of the step and refills its ids tensor before each replay (the reference rebuilds its segment
+        tensors once per forward, valora/server/router/model_infer/model_rpc.py:381)."""
+        if ids is not None:
+            if ids.dtype != torch.long or ids.numel() != self.T or ids.device != self.device:
+                raise RuntimeError(f"rebuild takes {self.T} int64 ids on {self.device}")
+            self._keep = (ids.contiguous(),) + self._keep[1:]
+        ids, a_start, a_len = self._keep
+        _lib.check(_lib.lib().mlora_build_plan(_lib.current_stream(self.device), self.handle, _lib.ptr(ids), self.T,
+                                               _lib.ptr(a_start), _lib.ptr(a_len), self.n_adapters, self.n_slots,
+                                               self.bm_shrink, self.bm_expand))
 
     # -- introspection (synchronises; for tests and diagnostics) --------------------------------
     def header(self) -> dict:
