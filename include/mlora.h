@@ -54,9 +54,14 @@ enum {
                                  two-launch op with
                                  MLORA_REDUCE_IN_EXPAND and the same ksplit.  Launches that share a plan
                                  must not overlap in time.                                        */
-  MLORA_ONE_LAUNCH_NO_WAIT = 4 /* with MLORA_ONE_LAUNCH: expand items do not wait at all and always
+  MLORA_ONE_LAUNCH_NO_WAIT = 4, /* with MLORA_ONE_LAUNCH: expand items do not wait at all and always
                                  compute their tile's partials themselves (the give-up path made
                                  testable; same results, slower)                                  */
+  MLORA_SHRINK_RECOMPUTE = 8  /* a split-K shrink of a small batch (tiles up to 64 tokens) sums its K
+                                 chunks inside the launch: the chunk of a tile that finishes last reads
+                                 the others' partials out of the L2 it shares with them, or -- when they
+                                 did not all run on its XCD -- computes them itself.  This flag makes
+                                 every tile take the second path (made testable; same results, slower) */
 };
 
 /* What the kernels can vary per batch shape (see mlora_tile_lookup). */

@@ -33,7 +33,9 @@ def test_size_queries():
     L = _lib.lib()
     assert L.mlora_plan_bytes(0, 0) > 0
     assert L.mlora_plan_bytes(256, 64) >= (32 + 3 * 256 + 2 * 8 * (16 + 64) + 4 * 64) * 4
-    assert L.mlora_scratch_bytes(256, 16, 8) == 256 * 16 * 2 + 8 * 256 * 16 * 4   # v (T) + fp32 partials
+    # v (T) + fp32 partials, whose rows are whole 128-byte lines (32 floats for rank 16)
+    assert L.mlora_scratch_bytes(256, 16, 8) == 256 * 16 * 2 + 8 * 256 * 32 * 4
+    assert L.mlora_scratch_bytes(256, 64, 8) == 256 * 64 * 2 + 8 * 256 * 64 * 4
     assert L.mlora_scratch_bytes(16, 8, 1) == 16 * 16 * 2       # rows padded to 16 columns, no partials
     assert L.mlora_workspace_bytes(256, 64, 16) > L.mlora_plan_bytes(256, 64)
     assert L.mlora_plan_bytes(-1, 3) == 0

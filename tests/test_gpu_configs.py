@@ -157,6 +157,80 @@ def test_full_configs_gemm_shrink_tiles(dev, n, name):
                           f"config{n}/{name}/plan bm=128 ks={ks} reduce_in_expand={rie}")
 
 
+def _small_batches():
+    """Batches whose split-K shrink sums its chunks inside the launch (tiles up to 64 tokens, T <= 1024)."""
+    yield "config2", W.config2(), "q", (16, 32), (2, 4, 7)
+    yield "config1", W.config1(), "q", (16, 32, 64), (2, 8)
+    yield "config5/2", W.config5_layer(len_div=2, targets=("o",)), "o", (16,), (3, 8)
+    yield "config5/2 down", W.config5_layer(len_div=2, targets=("down",)), "down", (16, 32), (2, 4)
+    yield "config3/8", W.config3(len_div=8, targets=("q",)), "q", (16, 32, 64), (2, 5)
+
+
+def test_split_k_summed_in_the_shrink_launch(dev):
+    """Small batches with split-K and a shrink that has to deliver v itself: the chunk of a tile that finishes
+    last sums the partials out of the L2 -- or, when the chunks did not share an XCD (forced here by a flag),
+    computes them all itself.  Same bits both ways, on a plan that is used launch after launch (the arrival
+    words must be back at zero), and the same bits as the reduce launch gives (reached with tiles of 128)."""
+    from valora_amd.plan import LoraPlan
+    for label, w, name, bms, kss in _small_batches():
+        wd = w.to(dev)
+        want = oracle_target(w, name)
+        t = wd.target(name); p = t.pool
+        for bm in bms:
+            for ks in kss:
+                outs = []
+                for recompute in (False, True):
+                    plan = LoraPlan(wd.ids, p.a_start, p.a_len, max(p.ranks), hidden=t.h_in, bm_shrink=bm, ksplit=ks,
+                                    bm_expand=32, reduce_in_expand=False, shrink_recompute=recompute)
+                    for rep in range(1 if recompute else 3):
+                        y = wd.y0[name].clone()
+                        plan.apply(y, wd.x[t.h_in], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot,
+                                   p.a_scaling)
+                        outs.append(y)
+                # the expand that sums the chunks itself adds them in the same order
+                outs.append(run_plan(wd, name, bm_shrink=bm, ksplit=ks, bm_expand=32, reduce_in_expand=True))
+                for o in outs[1:]:
+                    assert torch.equal(o, outs[0]), f"{label}/{name} bm={bm} ks={ks}: the ways of summing the chunks differ"
+                assert_parity(outs[0].cpu(), want, f"{label}/{name}/split-K summed in the shrink, bm={bm} ks={ks}")
+
+
+def test_split_k_summed_in_the_shrink_launch_multi_target_and_token_order(dev):
+    """The same through apply_multi (q, k, v share x; arrival words per target) and through the entry point
+    that writes the caller's [T, r] matrix in token order (dispatch_bgmv's shrink)."""
+    w = W.config5_layer(len_div=2, targets=("q", "k", "v"))
+    wd = w.to(dev)
+    names = ("q", "k", "v")
+    kw = dict(bm_shrink=16, ksplit=5, bm_expand=32, reduce_in_expand=False)
+    ys = run_multi(wd, names, **kw)
+    ys2 = run_multi(wd, names, shrink_recompute=True, **kw)
+    for name, y, y2 in zip(names, ys, ys2):
+        assert torch.equal(y, y2)
+        assert torch.equal(y, run_plan(wd, name, **kw))
+        assert_parity(y.cpu(), oracle_target(w, name), f"config5/2 {name}/multi, split-K summed in the shrink")
+    from valora_amd import _lib
+    from valora_amd.plan import LoraPlan
+    w2 = W.config2()
+    wd2 = w2.to(dev)
+    t = wd2.target("q"); p = t.pool
+    L = _lib.lib()
+    R = max(p.ranks)
+    got = []
+    for flags in (0, _lib.SHRINK_RECOMPUTE):
+        plan = LoraPlan(wd2.ids, p.a_start, p.a_len, R, hidden=t.h_in, bm_shrink=16, ksplit=4, bm_expand=16)
+        delta = torch.full((w2.T, R), 7.0, dtype=w2.dtype, device=dev)
+        pa = _lib.make_pool(p.key_buffer, p.a_start, p.a_len, p.a_loc, t.h_in, 4)
+        for rep in range(2):
+            _lib.check(L.mlora_shrink(_lib.current_stream(dev), plan.handle, _lib.ptr(plan.scratch), plan.scratch.numel(),
+                                      _lib.ptr(wd2.x[t.h_in]), w2.T, t.h_in, R, pa, t.slot, 4, _lib.ptr(delta), R, 0, 0, flags,
+                                      _lib.dtype_code(w2.dtype)))
+        got.append(delta)
+    assert torch.equal(got[0], got[1])
+    pc = w2.target("q").pool
+    want = O.bgmv_shrink(torch.full((w2.T, R), 7.0, dtype=w2.dtype), w2.x[t.h_in], pc.key_buffer, pc.a_start, pc.a_len,
+                         pc.a_loc, w2.ids, t.slot)
+    assert_parity(got[0].cpu(), want, "config2/q shrink in token order, split-K summed in the launch")
+
+
 @pytest.mark.parametrize("n,names", [(3, ("q", "k", "v")), (4, ("gate", "up")), (5, ("q", "k", "v"))])
 def test_full_configs_multi_target(dev, n, names):
     w = W.CONFIGS[n]()

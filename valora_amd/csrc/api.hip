@@ -99,7 +99,8 @@ int check_dims(int64_t T, int64_t wide, int64_t narrow, int64_t h_in, int64_t h_
 size_t scratch_bytes(int64_t T, int64_t max_rank, int ksplit) {
   const int64_t rp = partial_stride(max_rank);
   size_t n = (size_t)align_up(T * rp * 2, 256);
-  if (ksplit > 1) n += (size_t)ksplit * (size_t)T * (size_t)rp * 4;
+  // the partials' rows are whole 128-byte lines when the shrink sums them itself (128-token tiles)
+  if (ksplit > 1) n += (size_t)ksplit * (size_t)T * (size_t)partial_stride_lines(max_rank) * 4;
   return n < 256 ? 256 : n;
 }
 
@@ -112,6 +113,20 @@ PoolDev pool_dev(const mlora_pool *p) {
   d.a_loc = p->a_loc;
   d.a_loc_len = p->a_loc_len;
   return d;
+}
+
+// Small tiles (direct-load shrink, up to 64 tokens) of small batches sum their K chunks inside the launch: the
+// last chunk of a tile to finish reads the others' partials out of the L2 they share.  One workgroup then reads
+// ksplit x tile x rank x 4 bytes at L2 latency, which beats a separate reduce launch (about 3.7 us with the gap
+// between the launches) only while that is a few tens of KB; the 128-token tiles and large batches keep the
+// reduce launch (or leave the sum to the expand).
+void set_reduce_here(ShrinkArgs &a, const mlora_plan *plan, const PlanLayout &L, int64_t max_rank, int flags) {
+  const int64_t tile_bytes = (int64_t)a.ksplit * plan->bm_shrink * partial_stride_lines(max_rank) * 4;
+  const bool small = plan->bm_shrink <= 64 && tile_bytes <= 32768 && plan->T <= 1024;
+  a.reduce_here = (small && a.ksplit > 1 && !a.partial_only) ? ((flags & MLORA_SHRINK_RECOMPUTE) ? 2 : 1) : 0;
+  a.prp = (int)partial_stride_lines(max_rank);
+  a.n_tiles = (int)tiles_upper(plan->T, plan->n_adapters, plan->bm_shrink);
+  a.arrive = reinterpret_cast<unsigned long long *>(static_cast<int32_t *>(plan->dev) + L.off_stamps);
 }
 
 struct Carver {
@@ -283,10 +298,11 @@ int mlora_shrink(void *stream, const mlora_plan *plan, void *scratch, size_t scr
     a.width = 0;
     a.ncols = (int)rp;
   }
+  set_reduce_here(a, plan, L, max_rank, flags);
   if (int rc = launch_shrink((hipStream_t)stream, a, plan->bm_shrink, (int)max_rank,
                              tiles_upper(T, plan->n_adapters, plan->bm_shrink), dtype))
     return rc;
-  if (ksplit > 1 && !a.partial_only) return launch_shrink_reduce((hipStream_t)stream, a, dtype);
+  if (ksplit > 1 && !a.partial_only && !a.reduce_here) return launch_shrink_reduce((hipStream_t)stream, a, dtype);
   return MLORA_OK;
 }
 
@@ -448,11 +464,12 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
   for (int i = 0; i < MLORA_MAX_TARGETS; ++i) a.slots[i] = targets[i < n_targets ? i : 0].slot;
   a.out_tstride = (int64_t)(per_target / 2);
   a.partial_tstride = (int64_t)(per_target / 4);
+  set_reduce_here(a, plan, L, max_rank, flags);
   if (!use_decode) {
     if (int rc = launch_shrink((hipStream_t)stream, a, plan->bm_shrink, (int)max_rank,
                                tiles_upper(T, plan->n_adapters, plan->bm_shrink), dtype))
       return rc;
-    if (ksplit > 1 && !rie)
+    if (ksplit > 1 && !rie && !a.reduce_here)
       if (int rc = launch_shrink_reduce((hipStream_t)stream, a, dtype)) return rc;
   }
 

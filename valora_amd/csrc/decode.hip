@@ -69,8 +69,6 @@ __device__ __forceinline__ bool stamps_match(const uint32_t *stamps, int n, uint
 }
 // workgroup barrier that orders LDS traffic only: outstanding global loads stay in flight across it
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-// which of the device's XCDs this wave runs on (bits 3:0 of the XCC_ID hardware register)
-__device__ __forceinline__ uint32_t xcd_id() { return (uint32_t)__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20); }
 
 __device__ __forceinline__ uint32_t stamp_of(uint32_t tag, uint32_t xcd) { return ((tag + 1u) << 4) | xcd; }
 

@@ -120,6 +120,9 @@ struct Traits<__bf16> {
   }
 };
 
+// which of the device's XCDs this wave runs on (bits 3:0 of the XCC_ID hardware register)
+__device__ __forceinline__ uint32_t xcd_id() { return (uint32_t)__builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20); }
+
 // 8 packed T values <-> 8 floats
 template <typename T>
 __device__ __forceinline__ void unpack8(u32x4 v, float (&f)[8]) {

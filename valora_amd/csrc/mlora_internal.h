@@ -16,7 +16,9 @@ namespace mlora {
 // padapter[p] adapter of position p;  prank[p] its rank
 // tile        {adapter, rank, first position, token count, a_start[adapter], 0, 0, 0}
 // done, stamps  the hand-off words of the one-launch op (csrc/decode.hip): per tile a count of the shrink items
-//             that have finished on this plan, and one stamp per shrink item; zeroed by the plan kernel
+//             that have finished on this plan, and one stamp per shrink item; zeroed by the plan kernel.
+//             The stamps of tile t also serve as the arrival words of the shrink's own split-K sum
+//             (csrc/shrink.hip), 8 x 64 bits per tile, zero between launches
 constexpr int HDR_WORDS = 32;
 constexpr int TILE_WORDS = 8;
 constexpr int32_t PLAN_MAGIC = 0x4d4c5241;
@@ -62,6 +64,9 @@ static inline int64_t tiles_upper(int64_t T, int64_t A, int bm) {
 }
 
 static inline int64_t partial_stride(int64_t max_rank) { return align_up(max_rank, 16); }
+// row stride of the split-K partials when the shrink sums them itself: every row owns whole 128-byte lines, so
+// no line holds rows of two tiles
+static inline int64_t partial_stride_lines(int64_t max_rank) { return align_up(max_rank, 32); }
 
 // ---- error reporting (api.hip) ---------------------------------------------------------------
 int fail(int code, const char *fmt, ...);
@@ -96,6 +101,11 @@ struct ShrinkArgs {
   int n_targets;
   int slots[MLORA_MAX_TARGETS];
   int64_t out_tstride, partial_tstride;   // elements / floats between consecutive targets
+  // split-K summed inside the launch by the last K chunk of a tile to arrive (small tiles, csrc/shrink.hip)
+  int reduce_here;            // 0 off, 1 on, 2 on with every sum taking the recompute path (tests)
+  int prp;                    // row stride of the partials in that mode: whole 128-byte lines per row
+  int n_tiles;                // upper bound of the tile count
+  unsigned long long *arrive; // [tiles][MLORA_MAX_TARGETS * 2] arrival words, zero between launches
 };
 
 struct ExpandArgs {

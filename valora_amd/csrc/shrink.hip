@@ -55,10 +55,7 @@ __device__ __forceinline__ void store_v(const ShrinkArgs &p, int pos, int t, int
 //   ksplit  > 1 : stored as this K-chunk's fp32 partial (ordinary stores, then the workgroup is
 //                 done); a later launch on the stream -- shrink_reduce_kernel, or the expand
 //                 itself for small batches -- sums the chunks in index order and rounds once.
-// An in-kernel hand-off (last workgroup of a tile sums the chunks, found through an atomic
-// counter) was measured and dropped: on this multi-XCD part it needs device-scope stores, an
-// atomic and device-scope loads, i.e. three to four dependent memory round trips at the end of
-// every workgroup (+14 us on a 30 us kernel); a device-scope fence instead made it 5-10x slower.
+// (shrink_kernel can also sum the chunks itself, see there.)
 template <typename T>
 __device__ __forceinline__ void shrink_epilogue(const ShrinkArgs &p, const float *tile, int ld, int s, int pos0,
                                                 int cnt, int r, const int32_t *perm) {
@@ -112,15 +109,29 @@ __global__ __launch_bounds__(256) void shrink_reduce_kernel(ShrinkArgs args_in) 
 
 template <typename T, int MB, int NB>
 __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs args_in) {
-  // workgroup id = (tile * targets + target) * ksplit + K chunk.  The id mod 8 selects the XCD, so
-  // with the K chunk as the fast index the tiles of an adapter that share a K chunk of A, and the
-  // targets that share a K chunk of x, meet in one L2.
-  const int wg_tz = blockIdx.x / args_in.ksplit;
-  const int tile_idx = wg_tz / args_in.n_targets;
-  const ShrinkArgs p = select_target(args_in, wg_tz - tile_idx * args_in.n_targets);
-  const int s = blockIdx.x - wg_tz * p.ksplit;
+  int tile_idx, z_idx, s;
+  if (args_in.reduce_here) {
+    // The K chunks of a tile are summed by whichever of them finishes last, out of the L2 they share: the id
+    // mod 8 selects the XCD, so all chunks (and targets) of a tile get ids that agree mod 8.
+    const int per_tile = args_in.n_targets * args_in.ksplit;
+    const int local = blockIdx.x >> 3, tl = local / per_tile, rem = local - tl * per_tile;
+    tile_idx = tl * 8 + (blockIdx.x & 7);
+    z_idx = rem / args_in.ksplit;
+    s = rem - z_idx * args_in.ksplit;
+    if (tile_idx >= args_in.n_tiles) return;
+  } else {
+    // workgroup id = (tile * targets + target) * ksplit + K chunk.  The id mod 8 selects the XCD, so
+    // with the K chunk as the fast index the tiles of an adapter that share a K chunk of A, and the
+    // targets that share a K chunk of x, meet in one L2.
+    const int wg_tz = blockIdx.x / args_in.ksplit;
+    tile_idx = wg_tz / args_in.n_targets;
+    z_idx = wg_tz - tile_idx * args_in.n_targets;
+    s = blockIdx.x - wg_tz * args_in.ksplit;
+  }
+  const ShrinkArgs p = select_target(args_in, z_idx);
   constexpr int NBLK = MB * NB;
   __shared__ float red[2][NBLK * 256];
+  __shared__ int s_last;
 
   const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
@@ -129,7 +140,89 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs args_in) {
   const int kbeg = s * p.kchunk;
   const int kend = min(p.h_in, kbeg + p.kchunk);
   shrink_tile_to_lds<T, MB, NB>(p.x, p.h_in, p.pool, p.slot, perm, r, pos0, cnt, astart, kbeg, kend, red);
-  shrink_epilogue<T>(p, red[1], NB * 16, s, pos0, cnt, r, perm);
+  if (!p.reduce_here || p.ksplit == 1) {
+    shrink_epilogue<T>(p, red[1], NB * 16, s, pos0, cnt, r, perm);
+    return;
+  }
+
+  // ---- split-K summed here: every chunk leaves its partial in the L2, the last one to arrive adds them up.
+  // Partials are plain stores into rows that own whole 128-byte lines (prp floats per row), so a line never
+  // holds rows of two tiles and no compute unit has read it before the tile is complete.  A chunk announces
+  // itself -- after its stores have been acknowledged by the L2 -- by adding to the tile's arrival word (one
+  // atomic per workgroup, device scope): the count in the low byte, and one more count in the field of the XCD
+  // it runs on.  Whoever brings the count to ksplit is the last: it knows all partials are written, and from
+  // its XCD's field whether all of them were written through ITS L2.  If so it reads them back (L2 hits) and
+  // sums them in index order; if not (the workgroups of the tile were not placed the way the id layout
+  // expects) it computes every chunk itself, in the same order with the same code: same bits, no waiting
+  // anywhere, and nothing depends on where or when a workgroup runs.  It then puts the word back to zero for
+  // the next launch on this plan (launches that share a plan must not overlap).
+  // (Worth it for small tiles only: one workgroup reads ksplit x tile x prp x 4 bytes at L2 latency.  For
+  // 128-token tiles of rank 64 that is 256 KB and measured 8.5 us, against 3.7 us for the reduce launch.)
+  const int tid = threadIdx.x;
+  const int quarter = p.rp >> 2, pq = p.prp >> 2;
+  {
+    f32x4 *part = reinterpret_cast<f32x4 *>(p.partial + ((int64_t)s * p.T + pos0) * p.prp);
+    for (int e = tid; e < cnt * quarter; e += 256) {
+      const int row = e / quarter, c4 = e - row * quarter;
+      const float *src = red[1] + row * (NB * 16) + 4 * c4;
+      part[row * pq + c4] = f32x4{src[0], src[1], src[2], src[3]};
+    }
+  }
+  wait_vmcnt<0>();
+  __syncthreads();
+  if (tid == 0) {
+    const uint32_t xcd = xcd_id();
+    unsigned long long *word = p.arrive + (int64_t)tile_idx * (2 * MLORA_MAX_TARGETS) + z_idx;
+    const unsigned long long add = 1ull + (xcd < 8 ? 1ull << (8 + 7 * xcd) : 0ull);
+    const unsigned long long now = __hip_atomic_fetch_add(word, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + add;
+    int last = 0;
+    if ((int)(now & 0xffull) == p.ksplit) {
+      const bool all_here = xcd < 8 && (int)((now >> (8 + 7 * xcd)) & 0x7full) == p.ksplit;
+      last = (all_here && p.reduce_here == 1) ? 1 : 2;
+      __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    s_last = last;
+  }
+  __syncthreads();
+  const int last = s_last;
+  if (last == 0) return;
+  if (last == 1) {
+    // v[row, :] = T(0 + p_0 + p_1 + ...): the order shrink_reduce_kernel uses
+    const f32x4 *src = reinterpret_cast<const f32x4 *>(p.partial + (int64_t)pos0 * p.prp);
+    const int64_t sstride = (int64_t)p.T * pq;
+    for (int e = tid; e < cnt * quarter; e += 256) {
+      const int row = e / quarter, c4 = e - row * quarter;
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      for (int s0 = 0; s0 < p.ksplit; s0 += 8) {
+        f32x4 q[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          q[u] = (s0 + u < p.ksplit) ? src[(s0 + u) * sstride + row * pq + c4] : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v += q[u];
+      }
+      const int t = p.out_by_token ? perm[pos0 + row] : 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) store_v<T>(p, pos0 + row, t, r, 4 * c4 + i, v[i]);
+    }
+    return;
+  }
+  // the chunks were not all written through this XCD's L2 (or the caller asked for this path): compute them
+  // here, one after the other, and add them up in LDS
+  __shared__ float vacc[16 * MB * NB * 16];
+  for (int e = tid; e < 16 * MB * NB * 16; e += 256) vacc[e] = 0.f;
+  for (int c = 0; c < p.ksplit; ++c) {
+    const int kb = c * p.kchunk;
+    __syncthreads();
+    shrink_tile_to_lds<T, MB, NB>(p.x, p.h_in, p.pool, p.slot, perm, r, pos0, cnt, astart, kb, min(p.h_in, kb + p.kchunk),
+                                  red);
+    for (int e = tid; e < 16 * MB * NB * 16; e += 256) vacc[e] += red[1][e];
+  }
+  __syncthreads();
+  for (int e = tid; e < cnt * p.rp; e += 256) {
+    const int row = e / p.rp, col = e - row * p.rp;
+    store_v<T>(p, pos0 + row, p.out_by_token ? perm[pos0 + row] : 0, r, col, vacc[row * (NB * 16) + col]);
+  }
 }
 
 // Prefill-sized tiles (128 tokens): GEMM structure with a three-stage LDS ring.
@@ -366,6 +459,7 @@ int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int
   nb = nb <= 1 ? 1 : nb <= 2 ? 2 : nb <= 4 ? 4 : 8;
   if (nb == 8 && bm == 64) return fail(MLORA_ERR_NO_KERNEL, "shrink: rank > 64 needs tile height 16, 32 or 128");
   if (grid_tiles <= 0) return MLORA_OK;
+  if (a.reduce_here) grid_tiles = (grid_tiles + 7) / 8 * 8;   // ids are dealt to the 8 XCDs tile by tile
   if (grid_tiles * a.ksplit * a.n_targets > 0x7fffffff) return fail(MLORA_ERR_NO_KERNEL, "shrink: grid too large");
   dim3 grid((unsigned)(grid_tiles * a.ksplit * a.n_targets));
   return dt == MLORA_F16 ? launch_shrink_t<_Float16>(st, a, bm, nb, grid)

@@ -23,13 +23,14 @@ class LoraPlan:
                  n_slots: int = 4, hidden: int = 4096, bm_shrink: Optional[int] = None,
                  bm_expand: Optional[int] = None, ksplit: Optional[int] = None,
                  reduce_in_expand: Optional[bool] = None, one_launch: Optional[bool] = None,
-                 one_launch_no_wait: bool = False):
+                 one_launch_no_wait: bool = False, shrink_recompute: bool = False):
         """``ids``: int64 per-token adapter index (negative = no adapter); ``a_start`` / ``a_len``:
         the pool index (``a_len = n_slots * rank``); ``max_rank``: widest rank among the resident
         adapters (the reference's ``max_lora_dim``, lora_unordered_batch_infer.py:181-182).
         ``one_launch``: shrink and expand as work items of one grid (decode-like batches; forces
         16-token tiles, needs ``max_rank <= 64``); ``None`` takes the tile table's choice.
-        ``one_launch_no_wait`` makes every expand item take its give-up path (tests)."""
+        ``one_launch_no_wait`` makes every expand item take its give-up path, ``shrink_recompute`` makes the
+        128-token shrink sum its K chunks by computing them all in one workgroup (both for tests)."""
         if not ids.is_cuda:
             raise RuntimeError("ids must be a CUDA tensor")
         if ids.dtype != torch.long or a_start.dtype != torch.long or a_len.dtype != torch.long:
@@ -54,6 +55,8 @@ class LoraPlan:
             self.bm_shrink = self.bm_expand = 16
             self.ksplit = max(2, self.ksplit)
             self.flags = _lib.REDUCE_IN_EXPAND | _lib.ONE_LAUNCH | (_lib.ONE_LAUNCH_NO_WAIT if one_launch_no_wait else 0)
+        if shrink_recompute:
+            self.flags |= _lib.SHRINK_RECOMPUTE
         L = _lib.lib()
         nbytes = int(L.mlora_plan_bytes(self.T, self.n_adapters))
         self.buf = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=self.device)
