@@ -16,7 +16,8 @@ namespace mlora {
 
 namespace {
 
-constexpr int PLAN_THREADS = 1024;
+constexpr int PLAN_THREADS = 1024;   // large batches; decode-sized ones run with PLAN_THREADS_SMALL
+constexpr int PLAN_THREADS_SMALL = 256;
 constexpr int PLAN_WAVES = PLAN_THREADS / 64;
 constexpr int HIST_WORDS = 8192;  // LDS words for the per-wave histograms
 
@@ -29,22 +30,52 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane) {
   return v;
 }
 
-// exclusive prefix of v over the 1024 threads; *total gets the block sum.
-__device__ __forceinline__ int block_exclusive_scan(int v, int *total, int *wsum /* LDS[17] */) {
+// exclusive prefix of v over the workgroup's threads (n_waves waves); *total gets the block sum.
+__device__ __forceinline__ int block_exclusive_scan(int v, int *total, int *wsum /* LDS[17] */, int n_waves = PLAN_WAVES) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int inc = wave_inclusive_scan(v, lane);
   __syncthreads();  // wsum may still be read from a previous scan
   if (lane == 63) wsum[wave] = inc;
   __syncthreads();
   if (wave == 0) {
-    int w = lane < PLAN_WAVES ? wsum[lane] : 0;
+    int w = lane < n_waves ? wsum[lane] : 0;
     int winc = wave_inclusive_scan(w, lane);
-    if (lane < PLAN_WAVES) wsum[lane] = winc - w;
-    if (lane == PLAN_WAVES - 1) wsum[PLAN_WAVES] = winc;
+    if (lane < n_waves) wsum[lane] = winc - w;
+    if (lane == n_waves - 1) wsum[PLAN_WAVES] = winc;
   }
   __syncthreads();
   *total = wsum[PLAN_WAVES];
   return wsum[wave] + inc - v;
+}
+
+// The same for four counters at once (one pass of barriers instead of four).
+struct Quad {
+  int c, ts, te, g;
+};
+__device__ __forceinline__ Quad quad_add(Quad a, Quad b) { return Quad{a.c + b.c, a.ts + b.ts, a.te + b.te, a.g + b.g}; }
+__device__ __forceinline__ Quad quad_wave_inclusive_scan(Quad v, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    Quad n{__shfl_up(v.c, d, 64), __shfl_up(v.ts, d, 64), __shfl_up(v.te, d, 64), __shfl_up(v.g, d, 64)};
+    if (lane >= d) v = quad_add(v, n);
+  }
+  return v;
+}
+__device__ __forceinline__ Quad block_exclusive_scan4(Quad v, Quad *total, Quad *wsum /* LDS[17] */, int n_waves) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const Quad inc = quad_wave_inclusive_scan(v, lane);
+  if (lane == 63) wsum[wave] = inc;
+  __syncthreads();
+  if (wave == 0) {
+    const Quad w = lane < n_waves ? wsum[lane] : Quad{0, 0, 0, 0};
+    const Quad winc = quad_wave_inclusive_scan(w, lane);
+    if (lane < n_waves) wsum[lane] = Quad{winc.c - w.c, winc.ts - w.ts, winc.te - w.te, winc.g - w.g};
+    if (lane == n_waves - 1) wsum[PLAN_WAVES] = winc;
+  }
+  __syncthreads();
+  *total = wsum[PLAN_WAVES];
+  const Quad base = wsum[wave];
+  return Quad{base.c + inc.c - v.c, base.ts + inc.ts - v.ts, base.te + inc.te - v.te, base.g + inc.g - v.g};
 }
 
 constexpr int PLAN_SMALL_A = 2048;   // adapters whose per-adapter tables fit in LDS next to the histograms
@@ -52,14 +83,17 @@ constexpr int PLAN_SMALL_A = 2048;   // adapters whose per-adapter tables fit in
 // SMALL: the per-adapter tables (counts, group starts, tile offsets, ranks, a_start) live in LDS instead of
 // the plan's scratch area, so the dependent look-ups of the later phases (the binary search of the tile
 // lists above all) cost LDS latency instead of a global round trip each.
-template <bool SMALL>
-__global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
+// THREADS: 1024, or 256 for decode-sized batches (a few hundred tokens), where the barriers and scans of sixteen
+// waves cost more than the work they organise.
+template <bool SMALL, int THREADS>
+__global__ __launch_bounds__(THREADS) void plan_kernel(
     int32_t *__restrict__ plan, const int64_t *__restrict__ ids, const int64_t *__restrict__ a_start,
     const int64_t *__restrict__ a_len, int T, int A, int n_slots, int bm_s, int bm_e, int W,
     int64_t off_perm, int64_t off_padapter, int64_t off_prank, int64_t off_tiles_s,
     int64_t off_tiles_e, int64_t off_counters, int64_t off_scratch, int max_tiles, int n_flag_words) {
+  constexpr int N_WAVES = THREADS / 64;
   __shared__ int32_t whist[HIST_WORDS];
-  __shared__ int wsum[PLAN_WAVES + 1];
+  __shared__ Quad wsum[PLAN_WAVES + 1];
   __shared__ int s_maxrank;
   __shared__ int s_err;
 
@@ -83,27 +117,33 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
   };
   auto start_of = [&](int a) -> int64_t { return SMALL ? s_astart[a] : a_start[a]; };
 
-  for (int i = tid; i < W * A; i += PLAN_THREADS) whist[i] = 0;
-  for (int i = tid; i < n_flag_words; i += PLAN_THREADS) plan[off_counters + i] = 0;
-  if (SMALL) {
-    for (int a = tid; a < A; a += PLAN_THREADS) {
-      const int64_t r = a_len[a] / n_slots;
-      s_rank[a] = (r > 0 && (r & 7) == 0 && r <= MAX_RANK) ? (int)r : 0;
-      s_astart[a] = a_start[a];
-    }
-  }
-  if (tid == 0) { s_maxrank = 0; s_err = 0; }
-  __syncthreads();
-
   // token range of each of the W histogram waves (contiguous, multiple of 64)
   const int cw = (int)align_up((T + W - 1) / W, 64);
   const int t_beg = wave * cw;
   const int t_end = (wave < W) ? min(T, t_beg + cw) : 0;
 
+  // Every global load the set-up needs is requested before the first store: a wave gets its memory results in
+  // issue order, so a load queued behind the zero-fill below would wait for those stores as well.
+  const int64_t id0 = (t_beg + lane < t_end) ? ids[t_beg + lane] : -1;
+  int64_t len0 = 0, start0 = 0;
+  if (SMALL && tid < A) { len0 = a_len[tid]; start0 = a_start[tid]; }
+
+  for (int i = tid; i < W * A; i += THREADS) whist[i] = 0;
+  if (SMALL) {
+    for (int a = tid; a < A; a += THREADS) {
+      const int64_t r = (a == tid ? len0 : a_len[a]) / n_slots;
+      s_rank[a] = (r > 0 && (r & 7) == 0 && r <= MAX_RANK) ? (int)r : 0;
+      s_astart[a] = a == tid ? start0 : a_start[a];
+    }
+  }
+  if (tid == 0) { s_maxrank = 0; s_err = 0; }
+  __syncthreads();
+  for (int i = tid; i < n_flag_words; i += THREADS) plan[off_counters + i] = 0;
+
   // 1. per-wave histogram of valid tokens (the first 64 tokens of a wave stay in registers for step 3)
   int first_a = -1, first_r = 0;
   for (int t = t_beg + lane; t < t_end; t += 64) {
-    const int64_t a64 = ids[t];
+    const int64_t a64 = (t < t_beg + 64) ? id0 : ids[t];
     int a = -1, r = 0;
     if (a64 >= 0 && a64 < A) {
       r = rank_of((int)a64);
@@ -117,7 +157,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
   __syncthreads();
 
   // 2. per-adapter totals, group starts, tile offsets (each thread owns a run of adapters)
-  const int per = (A + PLAN_THREADS - 1) / PLAN_THREADS;
+  const int per = (A + THREADS - 1) / THREADS;
   const int a_beg = min(A, tid * per), a_endx = min(A, a_beg + per);
   int my_c = 0, my_ts = 0, my_te = 0, my_g = 0, my_maxr = 0;
   for (int a = a_beg; a < a_endx; ++a) {
@@ -132,11 +172,10 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
       my_maxr = max(my_maxr, rank_of(a));
     }
   }
-  int n_active, n_ts, n_te, n_g;
-  int pre_c = block_exclusive_scan(my_c, &n_active, wsum);
-  int pre_ts = block_exclusive_scan(my_ts, &n_ts, wsum);
-  int pre_te = block_exclusive_scan(my_te, &n_te, wsum);
-  (void)block_exclusive_scan(my_g, &n_g, wsum);
+  Quad tot;
+  const Quad pre = block_exclusive_scan4(Quad{my_c, my_ts, my_te, my_g}, &tot, wsum, N_WAVES);
+  const int n_active = tot.c, n_ts = tot.ts, n_te = tot.te, n_g = tot.g;
+  int pre_c = pre.c, pre_ts = pre.ts, pre_te = pre.te;
   if (my_maxr > 0) atomicMax(&s_maxrank, my_maxr);
   for (int a = a_beg; a < a_endx; ++a) {
     const int c = cnt[a];
@@ -170,8 +209,13 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
         if (r > 0) a = (int)a64;
       }
     }
+    // Lanes holding the same adapter get consecutive positions in lane order.  A prefill batch has one or two
+    // adapters per 64 tokens: a few rounds of "take the first unplaced lane's adapter and place all its lanes"
+    // finish the step.  A decode batch has almost as many adapters as tokens, and a round costs an LDS round
+    // trip: what is left after four rounds is placed by rank instead (lanes before me with my adapter, found
+    // with 64 uniform-lane reads).
     unsigned long long remaining = __ballot(a >= 0);
-    while (remaining) {
+    for (int round = 0; remaining && round < 4; ++round) {
       const int leader = __ffsll((long long)remaining) - 1;
       const int a0 = __shfl(a, leader, 64);
       const unsigned long long m = __ballot(a == a0);
@@ -188,6 +232,25 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
       __builtin_amdgcn_wave_barrier();
       remaining &= ~m;
     }
+    if (remaining) {   // wave-uniform
+      const bool mine = (remaining >> lane) & 1ull;
+      int before = 0, after = 0;
+      for (int d = 0; d < 64; ++d) {
+        const int other = __builtin_amdgcn_readlane(a, d);
+        before += (other == a && d < lane) ? 1 : 0;
+        after += (other == a && d > lane) ? 1 : 0;
+      }
+      if (mine) {
+        const int slot_idx = wave * A + a;
+        const int pos = whist[slot_idx] + before;
+        perm[pos] = t;
+        padapter[pos] = a;
+        prank[pos] = r;
+        __builtin_amdgcn_wave_barrier();            // every lane of the group has read the offset ...
+        if (after == 0) whist[slot_idx] = pos + 1;  // ... before its last lane moves it on
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
   }
   __syncthreads();
 
@@ -197,7 +260,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
     const int bm = pass ? bm_e : bm_s;
     const int32_t *toff = pass ? toff_e : toff_s;
     int32_t *tiles = plan + (pass ? off_tiles_e : off_tiles_s);
-    for (int i = tid; i < n_tiles; i += PLAN_THREADS) {
+    for (int i = tid; i < n_tiles; i += THREADS) {
       int lo = 0, hi = A;  // first adapter with toff > i
       while (lo < hi) {
         const int mid = (lo + hi) >> 1;
@@ -220,7 +283,7 @@ __global__ __launch_bounds__(PLAN_THREADS) void plan_kernel(
     // the kernels' grids are sized with the upper bound of the tile count: records past the last
     // tile say "no tokens", so a workgroup needs no second look-up to know that it has nothing to do
     const int upper = (T + bm - 1) / bm + min(A, T);
-    for (int i = n_tiles + tid; i < upper; i += PLAN_THREADS) {
+    for (int i = n_tiles + tid; i < upper; i += THREADS) {
       int32_t *tl = tiles + (int64_t)i * TILE_WORDS;
 #pragma unroll
       for (int k = 0; k < TILE_WORDS; ++k) tl[k] = 0;
@@ -314,16 +377,18 @@ int launch_plan(hipStream_t st, int32_t *plan, const PlanLayout &L, const int64_
   int W = A > 0 ? (int)(HIST_WORDS / A) : PLAN_WAVES;
   if (W > PLAN_WAVES) W = PLAN_WAVES;
   if (W < 1) return fail(MLORA_ERR_NO_KERNEL, "plan: more than %lld adapters", (long long)MAX_ADAPTERS);
-  if (A <= PLAN_SMALL_A)
-    hipLaunchKernelGGL(plan_kernel<true>, dim3(1), dim3(PLAN_THREADS), 0, st, plan, ids, a_start, a_len,
-                       (int)L.T, A, n_slots, bm_s, bm_e, W, L.off_perm, L.off_padapter, L.off_prank,
-                       L.off_tiles_s, L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles,
-                       (int)(L.off_scratch - L.off_counters));
-  else
-    hipLaunchKernelGGL(plan_kernel<false>, dim3(1), dim3(PLAN_THREADS), 0, st, plan, ids, a_start, a_len,
-                       (int)L.T, A, n_slots, bm_s, bm_e, W, L.off_perm, L.off_padapter, L.off_prank,
-                       L.off_tiles_s, L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles,
-                       (int)(L.off_scratch - L.off_counters));
+  // the histogram is spread over as many waves as there are, W <= waves of the workgroup
+  const bool few = L.T <= 1024 && A <= 512;
+  if (few && W > PLAN_THREADS_SMALL / 64) W = PLAN_THREADS_SMALL / 64;
+#define MLORA_LAUNCH_PLAN(SMALL, THREADS)                                                                          \
+  hipLaunchKernelGGL((plan_kernel<SMALL, THREADS>), dim3(1), dim3(THREADS), 0, st, plan, ids, a_start, a_len,      \
+                     (int)L.T, A, n_slots, bm_s, bm_e, W, L.off_perm, L.off_padapter, L.off_prank, L.off_tiles_s,  \
+                     L.off_tiles_e, L.off_counters, L.off_scratch, (int)L.max_tiles,                              \
+                     (int)(L.off_scratch - L.off_counters))
+  if (few) MLORA_LAUNCH_PLAN(true, PLAN_THREADS_SMALL);
+  else if (A <= PLAN_SMALL_A) MLORA_LAUNCH_PLAN(true, PLAN_THREADS);
+  else MLORA_LAUNCH_PLAN(false, PLAN_THREADS);
+#undef MLORA_LAUNCH_PLAN
   return check_launch("plan_kernel");
 }
 
