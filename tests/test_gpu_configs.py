@@ -158,12 +158,13 @@ def test_full_configs_gemm_shrink_tiles(dev, n, name):
 
 
 def _small_batches():
-    """Batches whose split-K shrink sums its chunks inside the launch (tiles up to 64 tokens, T <= 1024)."""
+    """Batches whose split-K shrink sums its chunks inside the launch (tiles up to 64 tokens with at most 64 KB of partials each, T <= 4096)."""
     yield "config2", W.config2(), "q", (16, 32), (2, 4, 7)
     yield "config1", W.config1(), "q", (16, 32, 64), (2, 8)
     yield "config5/2", W.config5_layer(len_div=2, targets=("o",)), "o", (16,), (3, 8)
     yield "config5/2 down", W.config5_layer(len_div=2, targets=("down",)), "down", (16, 32), (2, 4)
     yield "config3/8", W.config3(len_div=8, targets=("q",)), "q", (16, 32, 64), (2, 5)
+    yield "config5", W.config5_layer(targets=("q",)), "q", (16, 32), (8,)
 
 
 def test_split_k_summed_in_the_shrink_launch(dev):

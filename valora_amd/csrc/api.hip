@@ -118,11 +118,12 @@ PoolDev pool_dev(const mlora_pool *p) {
 // Small tiles (direct-load shrink, up to 64 tokens) of small batches sum their K chunks inside the launch: the
 // last chunk of a tile to finish reads the others' partials out of the L2 they share.  One workgroup then reads
 // ksplit x tile x rank x 4 bytes at L2 latency, which beats a separate reduce launch (about 3.7 us with the gap
-// between the launches) only while that is a few tens of KB; the 128-token tiles and large batches keep the
-// reduce launch (or leave the sum to the expand).
+// between the launches) only while that is a few tens of KB (64 KB: 1 us faster on a 1152-token batch; 256 KB,
+// the 128-token tiles at rank 64: 5 us slower); those and large batches keep the reduce launch (or leave the
+// sum to the expand).
 void set_reduce_here(ShrinkArgs &a, const mlora_plan *plan, const PlanLayout &L, int64_t max_rank, int flags) {
   const int64_t tile_bytes = (int64_t)a.ksplit * plan->bm_shrink * partial_stride_lines(max_rank) * 4;
-  const bool small = plan->bm_shrink <= 64 && tile_bytes <= 32768 && plan->T <= 1024;
+  const bool small = plan->bm_shrink <= 64 && tile_bytes <= 65536 && plan->T <= 4096;
   a.reduce_here = (small && a.ksplit > 1 && !a.partial_only) ? ((flags & MLORA_SHRINK_RECOMPUTE) ? 2 : 1) : 0;
   a.prp = (int)partial_stride_lines(max_rank);
   a.n_tiles = (int)tiles_upper(plan->T, plan->n_adapters, plan->bm_shrink);
