@@ -494,6 +494,14 @@ def bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, r
         ev_e, wall_e = time_graph(torch, fn, max(10, reps // 4), 3, False)
         legs[name] = {"graph_us_per_layer": round(ev_g * 1e3 / L, 3), "eager_us_per_layer": round(ev_e * 1e3 / L, 3),
                       "eager_host_us_per_layer": round(wall_e * 1e3 / L, 3)}
+    # the same pair when every call sorts the tokens and cuts the tiles itself (plan = NULL at the C ABI)
+    from valora_amd import _plan_cache
+    _plan_cache.set_enabled(False)
+    try:
+        ev_g, _ = time_graph(torch, bgmv_pair, max(10, reps // 4), 3, True)
+        legs["valora._kernels.dispatch_bgmv, no plan reuse"] = {"graph_us_per_layer": round(ev_g * 1e3 / L, 3)}
+    finally:
+        _plan_cache.set_enabled(True)
     out["dropin_pair"] = legs
     out["dropin_pair_is"] = ("shrink + expand of the config-2 op through the reference's own entry points (two calls per "
                              "layer, torch binding -> one C-ABI call each with the cached plan of the batch); graph = HIP "

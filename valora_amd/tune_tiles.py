@@ -152,8 +152,11 @@ def main():
         k = tt.key(n_tokens, rank, hidden, n_adapters)
         if args.one_launch:
             if k in entries and n_tokens <= 1024 and rank <= 64:
-                entries[k], two, one = tune_one_launch(dev, n_tokens, min(n_adapters, max(1, n_tokens)), rank, hidden,
-                                                       entries[k])
+                new, two, one = tune_one_launch(dev, n_tokens, min(n_adapters, max(1, n_tokens)), rank, hidden, entries[k])
+                # a protected entry was tuned on its real workload: the synthetic batch (which may not fit the
+                # device as one grid where the real one does) can add the mark there, never take it away
+                if not (k in table.get("protected", []) and entries[k].get("one_launch") and not new.get("one_launch")):
+                    entries[k] = new
                 print(f"{k:24s} two launches {two:.1f} us, one launch {one:.1f} us -> {entries[k]}  "
                       f"[{time.time() - t0:.0f} s]", flush=True)
                 torch.cuda.empty_cache()
@@ -165,6 +168,8 @@ def main():
         entries[k] = cfg
         print(f"{k:24s} {cfg}  {us:.1f} us/op  [{time.time() - t0:.0f} s]", flush=True)
         torch.cuda.empty_cache()
+        with open(args.out, "w") as f:      # after every shape: a long sweep that is cut short keeps what it has
+            json.dump(table, f, indent=1)
     with open(args.out, "w") as f:
         json.dump(table, f, indent=1)
     print("wrote", args.out)
