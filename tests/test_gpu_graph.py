@@ -61,3 +61,66 @@ def test_graph_replays_match_eager(dev, n, kw, names):
         for got, want in zip(ys, eager):
             assert torch.equal(got, want), f"replay {i}"
         assert torch.isfinite(junk)
+
+
+def test_entry_points_under_capture_and_rebuild(dev):
+    """The reference's entry points inside a HIP graph, the way a serving loop captures a step: the first call of
+    a new batch happens DURING the capture, so the plan's build is only recorded.  Such a plan serves that capture
+    alone: an eager call with the same tensors before the first replay must not find it (its tiles were never
+    cut), and the replays must keep working afterwards.  A step graph that refills its ids tensor with `copy_`
+    rebuilds the plan inside the graph on every replay (the version counter moved, and the build is a graph node)."""
+    from oracle import lora_oracle as O
+    from tests._util import assert_parity
+    from valora_amd import _plan_cache
+    from valora_amd.kernels import dispatch_bgmv
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(77)
+    T, H, R = 200, 1024, 16
+    pool = W.make_pool([16, 8, 16, 16, 8], H, H, dtype, g, True, std=0.05)
+    pd = pool.to(dev)
+    idx = (pd.a_start, pd.a_len, pd.a_loc)
+    ids_a = torch.randint(0, 5, (T,), generator=g)
+    ids_b = torch.randint(0, 5, (T,), generator=g)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    y0 = torch.randn(T, H, generator=g).to(dtype)
+    xd, ids_d = x.to(dev), ids_a.to(dev)
+    y_graph, y_eager = y0.to(dev), y0.to(dev)
+    delta = torch.zeros(T, R, dtype=dtype, device=dev)
+    delta2 = torch.zeros(T, R, dtype=dtype, device=dev)
+
+    def want(ids):
+        return O.lora_op(y0, x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, 2,
+                         pool.a_scaling)
+
+    def pair(y, d):
+        dispatch_bgmv(d, xd, pd.key_buffer, *idx, ids_d, 2, pd.a_scaling)
+        dispatch_bgmv(y, d, pd.value_buffer, *idx, ids_d, 2, pd.a_scaling)
+
+    _plan_cache.clear()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        m0 = _plan_cache.misses
+        with torch.cuda.graph(graph, stream=s):
+            pair(y_graph, delta)                     # first sight of this batch: the plan build is a graph node
+        assert _plan_cache.misses - m0 == 1
+        # eager, same tensors, before any replay: needs a plan of its own
+        pair(y_eager, delta2)
+        torch.cuda.synchronize()
+        assert _plan_cache.misses - m0 == 2, "a plan recorded into a capture must not serve eager calls"
+        assert_parity(y_eager.cpu(), want(ids_a), "eager call after a capture")
+        for rep in range(3):
+            y_graph.copy_(y0)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert_parity(y_graph.cpu(), want(ids_a), f"replay {rep}")
+            assert torch.equal(y_graph, y_eager)
+        # the next batch of the same size: refill the ids tensor the graph reads; the replay cuts the tiles again
+        ids_d.copy_(ids_b.to(dev))
+        y_graph.copy_(y0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_parity(y_graph.cpu(), want(ids_b), "replay after the ids were refilled")
+    torch.cuda.current_stream().wait_stream(s)

@@ -21,6 +21,7 @@
 // (for the current stream).
 #include <torch/extension.h>
 
+#include <c10/hip/HIPFunctions.h>
 #include <c10/hip/HIPStream.h>
 #include <hip/hip_runtime_api.h>
 
@@ -45,6 +46,7 @@ void check_rc(int rc) {
 }
 
 // ---- the cache ------------------------------------------------------------------------------------
+// Module state without locks: every entry point is called from Python with the GIL held.
 constexpr int KEY_TENSORS = 8, KEY_SCALARS = 8;
 
 struct Key {
@@ -204,7 +206,21 @@ mlora_pool make_pool(const at::Tensor &w, const at::Tensor &a_start, const at::T
   return p;
 }
 
-hipStream_t current_stream(const at::Tensor &t) { return c10::hip::getCurrentHIPStream(t.get_device()).stream(); }
+// The stream the call's kernels go to: PyTorch's current stream on the operands' device, which has to be the
+// current device (the library launches on the current device; the reference's binding has the same contract).
+hipStream_t current_stream(const at::Tensor &t) {
+  const auto dev = t.get_device();
+  if (dev != c10::hip::current_device())
+    raise("operands live on cuda:" + std::to_string(dev) + " but the current device is cuda:" +
+          std::to_string(c10::hip::current_device()) + " (use torch.cuda.device)");
+  return c10::hip::getCurrentHIPStream(dev).stream();
+}
+
+void check_same_device(const at::Tensor &ref, std::initializer_list<const at::Tensor *> ts) {
+  for (const at::Tensor *t : ts)
+    if (t->defined() && t->is_cuda() && t->get_device() != ref.get_device())
+      raise("all operands must live on one device");
+}
 
 at::Tensor device_bytes(size_t n, const at::Tensor &like) {
   return at::empty({(int64_t)std::max<size_t>(n, 256)}, like.options().dtype(at::kByte));
@@ -249,6 +265,7 @@ void dispatch_bgmv(const at::Tensor &y, const at::Tensor &x, const at::Tensor &w
                    const at::Tensor &a_len, const at::Tensor &a_loc, const at::Tensor &ids, int64_t qkvo,
                    const c10::optional<at::Tensor> &lora_scales) {
   check_common(y, x, w, a_start, a_len, a_loc, ids);
+  check_same_device(x, {&y, &w, &a_start, &a_len, &a_loc, &ids});
   const int64_t T = x.size(0), h_in = x.size(1), h_out = y.size(1);
   const mlora_dtype code = dtype_code(x);
   if ((int)code < 0 || y.scalar_type() != x.scalar_type() || w.scalar_type() != x.scalar_type() || h_in >= 65536 ||
@@ -293,6 +310,7 @@ void dispatch_sgmm(const at::Tensor &y, const at::Tensor &x, const at::Tensor &w
                    const c10::optional<at::Tensor> &tmp_d, int64_t num_problems, int64_t, int64_t, int64_t, int64_t,
                    int64_t, int64_t) {
   check_common(y, x, w, a_start, a_len, a_loc, ids);
+  check_same_device(x, {&y, &w, &a_start, &a_len, &a_loc, &ids, &output_counts, &start_ids});
   const int64_t T = x.size(0), h_in = x.size(1), h_out = y.size(1);
   const mlora_dtype code = dtype_code(x);
   if ((int)code < 0 || y.scalar_type() != x.scalar_type() || w.scalar_type() != x.scalar_type() || h_in >= 65536 ||
@@ -390,6 +408,11 @@ Entry *request_plan(hipStream_t stream, const at::Tensor &like, const mlora_pool
                   });
 }
 
+void check_requests(const at::Tensor &b_start_loc, const at::Tensor &b_seq_len, const at::Tensor &b_indicies) {
+  if (!b_start_loc.is_cuda() || !b_seq_len.is_cuda() || !b_indicies.is_cuda())
+    raise("b_start_loc, b_seq_len and b_indicies must be CUDA tensors");
+}
+
 void check_index(const at::Tensor &b_loc, const at::Tensor &b_lora_start, const at::Tensor &b_lora_ranks) {
   check_input(b_loc, "b_loc");
   check_input(b_lora_start, "b_lora_start");
@@ -413,6 +436,8 @@ void lora_get_qkvo_fwd_shrink(const at::Tensor &x, const at::Tensor &w, const at
     raise("x rows must be dense, o and w must have unit inner stride");
   if (!x.is_cuda() || !o.is_cuda() || !w.is_cuda()) raise("x, w and o must be CUDA tensors");
   check_index(b_loc, b_lora_start, b_lora_ranks);
+  check_requests(b_start_loc, b_seq_len, b_indicies);
+  check_same_device(x, {&w, &o, &b_loc, &b_lora_start, &b_lora_ranks, &b_start_loc, &b_seq_len, &b_indicies});
   const int64_t T = x.size(0);
   const mlora_pool pool = make_pool(w, b_lora_start, b_lora_ranks, b_loc, hidden_size);
   const hipStream_t stream = current_stream(x);
@@ -443,6 +468,8 @@ void lora_get_qkvo_fwd_expand(const at::Tensor &x, const at::Tensor &w, const at
     raise("o rows must be dense, x and w must have unit inner stride");
   if (!x.is_cuda() || !o.is_cuda() || !w.is_cuda() || !scale.is_cuda()) raise("x, w, o and scale must be CUDA tensors");
   check_index(b_loc, b_lora_start, b_lora_ranks);
+  check_requests(b_start_loc, b_seq_len, b_indicies);
+  check_same_device(x, {&w, &o, &scale, &b_loc, &b_lora_start, &b_lora_ranks, &b_start_loc, &b_seq_len, &b_indicies});
   const int64_t T = o.size(0);
   at::Tensor keep;
   const void *scales = scales_ptr(scale, x, keep);
