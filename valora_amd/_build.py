@@ -26,6 +26,9 @@ BINDING_PATH = os.path.join(HERE, "_binding.so")
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first 8 dwords of a kernel's scalar arguments arrive in registers instead of through a load of the
+    # argument block (decode_kernel puts what its first dependent loads need there)
+    "-mllvm", "-amdgpu-kernarg-preload-count=8",
     "-Wall", "-Wno-unused-function",
 ]
 

@@ -82,18 +82,18 @@ struct ItemId {
   bool shrink;
   int tile, item;
 };
-__device__ __forceinline__ ItemId item_of(const DecodeArgs &a, int id) {
+__device__ __forceinline__ ItemId item_of(int n_producers, int n_consumers, int groups_per_chunk, int id) {
   ItemId it;
-  const int per_group = 8 * (a.n_producers + a.n_consumers);
-  const int per_chunk = a.groups_per_chunk * per_group;
+  const int per_group = 8 * (n_producers + n_consumers);
+  const int per_chunk = groups_per_chunk * per_group;
   const int chunk = id / per_chunk, local = id - chunk * per_chunk;
-  const int n_shrink = a.groups_per_chunk * 8 * a.n_producers;
+  const int n_shrink = groups_per_chunk * 8 * n_producers;
   it.shrink = local < n_shrink;
   const int l2 = it.shrink ? local : local - n_shrink;
-  const int per = it.shrink ? a.n_producers : a.n_consumers;
+  const int per = it.shrink ? n_producers : n_consumers;
   const int q8 = l2 >> 3, g = q8 / per;
   it.item = q8 - g * per;
-  it.tile = (chunk * a.groups_per_chunk + g) * 8 + (l2 & 7);
+  it.tile = (chunk * groups_per_chunk + g) * 8 + (l2 & 7);
   return it;
 }
 
@@ -105,8 +105,14 @@ __device__ __forceinline__ ItemId item_of(const DecodeArgs &a, int id) {
 // chunk, these are the items of the tiles that do not exist, unless the batch is larger than the device.
 // 3 waves per SIMD = 3 workgroups per compute unit: an expand item keeps the B fragments and y rows of 512
 // columns in flight, a shrink item 8 K-steps of both operands.
+// The leading scalar parameters repeat what the first dependent loads need (the tile records, the `done` words, the
+// id layout): the library is built with kernel-argument preloading, which hands the first 8 dwords of the
+// argument list to the wave in registers at launch, so the tile record can be requested without waiting for a load
+// of the argument block first (0.35 us of a 10.3 us op).
 template <typename T, int NB>
-__global__ __launch_bounds__(256, 3) void decode_kernel(DecodeArgs a) {
+__global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_base, const uint32_t *done_base, int h_n_producers,
+                                                        int h_n_consumers, int h_groups_per_chunk, int h_n_tiles,
+                                                        int h_resident, DecodeArgs a) {
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   constexpr int KB = (NB + 1) / 2;                  // 32-wide rank blocks of the expand
@@ -120,22 +126,22 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(DecodeArgs a) {
   __shared__ int32_t s_ready;
   float(*red)[NB * 256] = reinterpret_cast<float(*)[NB * 256]>(s_buf);
   const int id = (int)blockIdx.x;
-  const bool on_time = id < a.resident;
+  const bool on_time = id < h_resident;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rp = a.s.rp;
   const int32_t *__restrict__ perm = a.s.plan + a.s.off_perm;
 
-  const ItemId it = item_of(a, id);
+  const ItemId it = item_of(h_n_producers, h_n_consumers, h_groups_per_chunk, id);
   const bool shrink_item = it.shrink;
   const int item = it.item, tile_idx = it.tile;
-  if (tile_idx >= a.n_tiles) return;
-  const int32_t *__restrict__ tile = a.s.plan + a.e.off_tiles + (int64_t)tile_idx * TILE_WORDS;
+  if (tile_idx >= h_n_tiles) return;
+  const int32_t *__restrict__ tile = tiles_base + (int64_t)tile_idx * TILE_WORDS;
   const int ad = tile[0], r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
   if (shrink_item && !on_time) return;
   // the launch's tag: what the tile's `done` word holds while none of this launch's shrink items has finished
-  const uint32_t want_stamp = stamp_of(a.done[tile_idx], xcd_id());
+  const uint32_t want_stamp = stamp_of(done_base[tile_idx], xcd_id());
   uint32_t *const stamps = a.stamps + (int64_t)tile_idx * DECODE_MAX_PRODUCERS;
   // a tile's partials: [target][K chunk][16 rows][rp] floats, whole lines of the tile's own
   float *const tile_partial = a.s.partial + (int64_t)tile_idx * a.n_producers * 16 * rp;
@@ -350,9 +356,9 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(DecodeArgs a) {
 template <typename T>
 int launch_decode_t(hipStream_t st, const DecodeArgs &a, int nb, dim3 grid) {
   switch (nb) {
-    case 1: hipLaunchKernelGGL((decode_kernel<T, 1>), grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((decode_kernel<T, 2>), grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL((decode_kernel<T, 4>), grid, dim3(256), 0, st, a); break;
+    case 1: hipLaunchKernelGGL((decode_kernel<T, 1>), grid, dim3(256), 0, st, a.s.plan + a.e.off_tiles, (const uint32_t *)a.done, a.n_producers, a.n_consumers, a.groups_per_chunk, a.n_tiles, a.resident, a); break;
+    case 2: hipLaunchKernelGGL((decode_kernel<T, 2>), grid, dim3(256), 0, st, a.s.plan + a.e.off_tiles, (const uint32_t *)a.done, a.n_producers, a.n_consumers, a.groups_per_chunk, a.n_tiles, a.resident, a); break;
+    case 4: hipLaunchKernelGGL((decode_kernel<T, 4>), grid, dim3(256), 0, st, a.s.plan + a.e.off_tiles, (const uint32_t *)a.done, a.n_producers, a.n_consumers, a.groups_per_chunk, a.n_tiles, a.resident, a); break;
     default: return fail(MLORA_ERR_NO_KERNEL, "one-launch op: ranks above 64 use the two-launch path");
   }
   return check_launch("decode_kernel");

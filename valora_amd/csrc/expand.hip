@@ -45,18 +45,21 @@ __device__ __forceinline__ ExpandArgs select_target(const ExpandArgs &a, int z) 
 constexpr int expand_min_waves(int kb, bool partial) { return (kb == 2 && !partial) ? 5 : 1; }
 
 template <typename T, int KB, bool PARTIAL>
-__global__ __launch_bounds__(256, expand_min_waves(KB, PARTIAL)) void expand_kernel(ExpandArgs args_in) {
-  const ExpandArgs p = select_target(args_in, blockIdx.y);
+__global__ __launch_bounds__(256, expand_min_waves(KB, PARTIAL)) void expand_kernel(const int32_t *tiles_base, int h_n_ochunks,
+                                                                                    ExpandArgs args_in) {
+  // (tiles_base, h_n_ochunks: what the first dependent load needs, in front so that kernel-argument preloading
+  // delivers them in registers)
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   __shared__ float stage[4][16][STAGE_LD];
   __shared__ int32_t s_perm[EXP_MAX_BM];
 
-  const int tile_idx = blockIdx.x / p.n_ochunks;
-  const int oc = blockIdx.x - tile_idx * p.n_ochunks;
-  const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
+  const int tile_idx = blockIdx.x / h_n_ochunks;
+  const int oc = blockIdx.x - tile_idx * h_n_ochunks;
+  const int32_t *__restrict__ tile = tiles_base + (int64_t)tile_idx * TILE_WORDS;
   const int a = tile[0], r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
+  const ExpandArgs p = select_target(args_in, blockIdx.y);
   const int rk = min(r, p.kmax);  // rank columns the narrow operand really has (bgmv_impl.cuh:167,186)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -207,16 +210,16 @@ template <typename T>
 int launch_expand_t(hipStream_t st, const ExpandArgs &a, int kb, dim3 grid) {
   switch (kb) {
     case 1:
-      if (a.partial) hipLaunchKernelGGL((expand_kernel<T, 1, true>), grid, dim3(256), 0, st, a);
-      else hipLaunchKernelGGL((expand_kernel<T, 1, false>), grid, dim3(256), 0, st, a);
+      if (a.partial) hipLaunchKernelGGL((expand_kernel<T, 1, true>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.n_ochunks, a);
+      else hipLaunchKernelGGL((expand_kernel<T, 1, false>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.n_ochunks, a);
       break;
     case 2:
-      if (a.partial) hipLaunchKernelGGL((expand_kernel<T, 2, true>), grid, dim3(256), 0, st, a);
-      else hipLaunchKernelGGL((expand_kernel<T, 2, false>), grid, dim3(256), 0, st, a);
+      if (a.partial) hipLaunchKernelGGL((expand_kernel<T, 2, true>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.n_ochunks, a);
+      else hipLaunchKernelGGL((expand_kernel<T, 2, false>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.n_ochunks, a);
       break;
     case 4:
-      if (a.partial) hipLaunchKernelGGL((expand_kernel<T, 4, true>), grid, dim3(256), 0, st, a);
-      else hipLaunchKernelGGL((expand_kernel<T, 4, false>), grid, dim3(256), 0, st, a);
+      if (a.partial) hipLaunchKernelGGL((expand_kernel<T, 4, true>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.n_ochunks, a);
+      else hipLaunchKernelGGL((expand_kernel<T, 4, false>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.n_ochunks, a);
       break;
     default: return fail(MLORA_ERR_NO_KERNEL, "expand: no kernel for %d rank blocks", kb);
   }

@@ -107,33 +107,36 @@ __global__ __launch_bounds__(256) void shrink_reduce_kernel(ShrinkArgs args_in) 
   }
 }
 
+// The leading scalar parameters repeat what the first dependent load (the tile record) needs: with kernel-argument
+// preloading they arrive in registers at launch, so that load does not wait for a load of the argument block.
 template <typename T, int MB, int NB>
-__global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs args_in) {
+__global__ __launch_bounds__(256) void shrink_kernel(const int32_t *tiles_base, int h_ksplit, int h_n_targets, int h_reduce_here,
+                                                     int h_n_tiles, ShrinkArgs args_in) {
   int tile_idx, z_idx, s;
-  if (args_in.reduce_here) {
+  if (h_reduce_here) {
     // The K chunks of a tile are summed by whichever of them finishes last, out of the L2 they share: the id
     // mod 8 selects the XCD, so all chunks (and targets) of a tile get ids that agree mod 8.
-    const int per_tile = args_in.n_targets * args_in.ksplit;
+    const int per_tile = h_n_targets * h_ksplit;
     const int local = blockIdx.x >> 3, tl = local / per_tile, rem = local - tl * per_tile;
     tile_idx = tl * 8 + (blockIdx.x & 7);
-    z_idx = rem / args_in.ksplit;
-    s = rem - z_idx * args_in.ksplit;
-    if (tile_idx >= args_in.n_tiles) return;
+    z_idx = rem / h_ksplit;
+    s = rem - z_idx * h_ksplit;
+    if (tile_idx >= h_n_tiles) return;
   } else {
     // workgroup id = (tile * targets + target) * ksplit + K chunk.  The id mod 8 selects the XCD, so
     // with the K chunk as the fast index the tiles of an adapter that share a K chunk of A, and the
     // targets that share a K chunk of x, meet in one L2.
-    const int wg_tz = blockIdx.x / args_in.ksplit;
-    tile_idx = wg_tz / args_in.n_targets;
-    z_idx = wg_tz - tile_idx * args_in.n_targets;
-    s = blockIdx.x - wg_tz * args_in.ksplit;
+    const int wg_tz = blockIdx.x / h_ksplit;
+    tile_idx = wg_tz / h_n_targets;
+    z_idx = wg_tz - tile_idx * h_n_targets;
+    s = blockIdx.x - wg_tz * h_ksplit;
   }
+  const int32_t *__restrict__ tile = tiles_base + (int64_t)tile_idx * TILE_WORDS;
   const ShrinkArgs p = select_target(args_in, z_idx);
   constexpr int NBLK = MB * NB;
   __shared__ float red[2][NBLK * 256];
   __shared__ int s_last;
 
-  const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
   const int r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
   const int32_t *__restrict__ perm = p.plan + p.off_perm;
@@ -238,14 +241,15 @@ __global__ __launch_bounds__(256) void shrink_kernel(ShrinkArgs args_in) {
 // later ds_read_b128 of an MFMA operand (16 rows, one chunk column) over the banks.  Two stages
 // are always in flight while the third is consumed; one s_barrier per K step.
 template <typename T, int NB>
-__global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
+__global__ __launch_bounds__(256) void shrink_gemm_kernel(const int32_t *tiles_base, int h_ksplit, int h_n_targets, int, int,
+                                                          ShrinkArgs args_in) {
   // workgroup id = (tile * targets + target) * ksplit + K chunk.  The id mod 8 selects the XCD, so
   // with the K chunk as the fast index the tiles of an adapter that share a K chunk of A, and the
   // targets that share a K chunk of x, meet in one L2.
-  const int wg_tz = blockIdx.x / args_in.ksplit;
-  const int tile_idx = wg_tz / args_in.n_targets;
-  const ShrinkArgs p = select_target(args_in, wg_tz - tile_idx * args_in.n_targets);
-  const int s = blockIdx.x - wg_tz * p.ksplit;
+  const int wg_tz = blockIdx.x / h_ksplit;
+  const int tile_idx = wg_tz / h_n_targets;
+  const ShrinkArgs p = select_target(args_in, wg_tz - tile_idx * h_n_targets);
+  const int s = blockIdx.x - wg_tz * h_ksplit;
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   constexpr int MBW = 2, KC = 64, KS = KC / 32, STAGES = 3;
@@ -260,7 +264,7 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
   constexpr int RING_BYTES = STAGES * STAGE_BYTES + 1024;   // + one scratch block for dummy loads
   __shared__ __align__(16) unsigned char s_raw[RING_BYTES > TILE_BYTES ? RING_BYTES : TILE_BYTES];
 
-  const int32_t *__restrict__ tile = p.plan + p.off_tiles + (int64_t)tile_idx * TILE_WORDS;
+  const int32_t *__restrict__ tile = tiles_base + (int64_t)tile_idx * TILE_WORDS;
   const int r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
   if (cnt <= 0) return;   // records past the last tile are zero
 
@@ -407,10 +411,10 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(ShrinkArgs args_in) {
 template <typename T>
 int launch_gemm_nb(hipStream_t st, const ShrinkArgs &a, int nb, dim3 grid) {
   switch (nb) {
-    case 1: hipLaunchKernelGGL((shrink_gemm_kernel<T, 1>), grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((shrink_gemm_kernel<T, 2>), grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL((shrink_gemm_kernel<T, 4>), grid, dim3(256), 0, st, a); break;
-    case 8: hipLaunchKernelGGL((shrink_gemm_kernel<T, 8>), grid, dim3(256), 0, st, a); break;
+    case 1: hipLaunchKernelGGL((shrink_gemm_kernel<T, 1>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
+    case 2: hipLaunchKernelGGL((shrink_gemm_kernel<T, 2>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
+    case 4: hipLaunchKernelGGL((shrink_gemm_kernel<T, 4>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
+    case 8: hipLaunchKernelGGL((shrink_gemm_kernel<T, 8>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
     default: return fail(MLORA_ERR_NO_KERNEL, "shrink: no kernel for rank blocks=%d", nb);
   }
   return check_launch("shrink_gemm_kernel");
@@ -419,10 +423,10 @@ int launch_gemm_nb(hipStream_t st, const ShrinkArgs &a, int nb, dim3 grid) {
 template <typename T, int MB>
 int launch_shrink_nb(hipStream_t st, const ShrinkArgs &a, int nb, dim3 grid) {
   switch (nb) {
-    case 1: hipLaunchKernelGGL((shrink_kernel<T, MB, 1>), grid, dim3(256), 0, st, a); break;
-    case 2: hipLaunchKernelGGL((shrink_kernel<T, MB, 2>), grid, dim3(256), 0, st, a); break;
-    case 4: hipLaunchKernelGGL((shrink_kernel<T, MB, 4>), grid, dim3(256), 0, st, a); break;
-    case 8: hipLaunchKernelGGL((shrink_kernel<T, (MB > 2 ? 2 : MB), 8>), grid, dim3(256), 0, st, a); break;
+    case 1: hipLaunchKernelGGL((shrink_kernel<T, MB, 1>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
+    case 2: hipLaunchKernelGGL((shrink_kernel<T, MB, 2>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
+    case 4: hipLaunchKernelGGL((shrink_kernel<T, MB, 4>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
+    case 8: hipLaunchKernelGGL((shrink_kernel<T, (MB > 2 ? 2 : MB), 8>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
     default: return fail(MLORA_ERR_NO_KERNEL, "shrink: no kernel for rank blocks=%d", nb);
   }
   return check_launch("shrink_kernel");
