@@ -27,7 +27,7 @@ int check_launch(const char *what) {
 }
 
 int expand_bn();
-int decode_bn();
+int decode_bn(int max_rank);   // output columns per expand item of the one-launch op
 
 // Polls of a tile's "ready" word before an expand item of the one-launch op stops waiting and computes the
 // tile's partials itself.  A poll is one memory round trip plus a short sleep (about a microsecond), the shrink
@@ -425,7 +425,7 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
   int decode_resident = 0;
   if (one_launch) {
     const int64_t groups8 = (tiles_upper(T, plan->n_adapters, 16) + 7) / 8 * 8;
-    const int64_t items = groups8 * ksplit * n_targets + groups8 * ((h_out + decode_bn() - 1) / decode_bn()) * n_targets;
+    const int64_t items = groups8 * ksplit * n_targets + groups8 * ((h_out + decode_bn((int)max_rank) - 1) / decode_bn((int)max_rank)) * n_targets;
     decode_resident = decode_resident_workgroups((int)max_rank, dtype);
     one_launch_fits = (flags & MLORA_ONE_LAUNCH_NO_WAIT) || (decode_resident > 0 && items * 4 <= (int64_t)decode_resident * 5);
   }
@@ -511,7 +511,7 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
     d.done = reinterpret_cast<uint32_t *>(words + L.off_counters);
     d.stamps = reinterpret_cast<uint32_t *>(words + L.off_stamps);
     d.n_tiles = (int)tiles;
-    d.e.n_ochunks = (int)((h_out + decode_bn() - 1) / decode_bn());
+    d.e.n_ochunks = (int)((h_out + decode_bn((int)max_rank) - 1) / decode_bn((int)max_rank));
     d.n_producers = ksplit * n_targets;
     d.n_consumers = d.e.n_ochunks * n_targets;
     d.groups_per_chunk = decode_resident / (8 * (d.n_producers + d.n_consumers));

@@ -45,9 +45,11 @@ namespace mlora {
 
 namespace {
 
-constexpr int DEC_CH = 2;          // 256-column chunks per expand item (fewer, fatter items: the whole grid
-                                   // should be resident at once, a waiting item holds its slot)
-constexpr int DEC_BN = 256 * DEC_CH;   // outputs per expand item
+// 256-column chunks per expand item: two (fewer, fatter items: the whole grid should be resident at once, a waiting
+// item holds its slot) up to rank 32; at rank 64 the B fragments of two chunks no longer fit the register budget of
+// three waves per SIMD (16 registers spilled), so those items take one chunk.
+constexpr int dec_ch(int nb) { return nb >= 4 ? 1 : 2; }
+constexpr int dec_nb(int max_rank) { return max_rank <= 16 ? 1 : max_rank <= 32 ? 2 : 4; }
 constexpr int DEC_WN = 64;         // outputs per wave and chunk
 constexpr int DEC_STAGE_LD = DEC_WN + 4;
 
@@ -115,6 +117,7 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
                                                         int h_resident, DecodeArgs a) {
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
+  constexpr int DEC_CH = dec_ch(NB), DEC_BN = 256 * DEC_CH;   // chunks and outputs per expand item
   constexpr int KB = (NB + 1) / 2;                  // 32-wide rank blocks of the expand
   constexpr int STAGE_FLOATS = 4 * 16 * DEC_STAGE_LD;
   constexpr int RED_FLOATS = 2 * NB * 256;          // cross-wave reduction of shrink_tile_to_lds
@@ -366,7 +369,7 @@ int launch_decode_t(hipStream_t st, const DecodeArgs &a, int nb, dim3 grid) {
 
 }  // namespace
 
-int decode_bn() { return DEC_BN; }
+int decode_bn(int max_rank) { return 256 * dec_ch(dec_nb(max_rank)); }
 
 // How many workgroups of decode_kernel the current device can hold at the same time (0 if the runtime cannot
 // tell).  The one-launch op is only used for grids that fit: an item that starts after its tile's shrink

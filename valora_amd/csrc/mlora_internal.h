@@ -144,7 +144,7 @@ struct DecodeArgs {
   int spin_limit;             // polls of a tile's stamps before an expand item computes the partials itself
 };
 int launch_decode(hipStream_t st, const DecodeArgs &a, int max_rank, mlora_dtype dt);
-int decode_bn();
+int decode_bn(int max_rank);   // output columns per expand item of the one-launch op
 int decode_resident_workgroups(int max_rank, mlora_dtype dt);   // workgroups of decode_kernel the current device holds at once
 size_t decode_partial_floats(int64_t n_tiles, int n_targets, int ksplit, int64_t rp);
 int launch_plan(hipStream_t st, int32_t *plan, const PlanLayout &L, const int64_t *ids,
