@@ -208,3 +208,38 @@ def test_one_launch_request_on_a_large_batch_runs_as_two_launches(dev):
     one.apply(a, wd.x[512], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
     two.apply(b, wd.x[512], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
     assert torch.equal(a, b)
+
+
+def test_one_launch_op_and_in_launch_split_k_sum_share_a_plan(dev):
+    """Through the C ABI nothing stops a caller from running the one-launch op and a stand-alone split-K shrink
+    (which sums its chunks inside the launch) on the same plan, in any order: their hand-off words are separate."""
+    from oracle import lora_oracle as O
+    from tests._util import assert_parity
+    from valora_amd import _lib
+    from valora_amd.plan import LoraPlan
+    L = _lib.lib()
+    w = W.config2(hidden=1024, n_tokens=96, n_adapters=24)
+    wd = w.to(dev)
+    t = wd.target("q"); p = t.pool
+    pc = w.target("q").pool
+    R = max(p.ranks)
+    plan = LoraPlan(wd.ids, p.a_start, p.a_len, R, hidden=t.h_in, one_launch=True, ksplit=4)
+    pa = _lib.make_pool(p.key_buffer, p.a_start, p.a_len, p.a_loc, t.h_in, 4)
+    code = _lib.dtype_code(w.dtype)
+    want_y = O.lora_op(w.y0["q"], w.x[t.h_in], pc.key_buffer, pc.value_buffer, pc.a_start, pc.a_len, pc.a_loc, w.ids, t.slot,
+                       pc.a_scaling)
+    want_d = O.bgmv_shrink(torch.zeros(w.T, R, dtype=w.dtype), w.x[t.h_in], pc.key_buffer, pc.a_start, pc.a_len, pc.a_loc,
+                           w.ids, t.slot)
+    first = None
+    for rep in range(3):
+        y = wd.y0["q"].clone()
+        plan.apply(y, wd.x[t.h_in], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
+        delta = torch.zeros(w.T, R, dtype=w.dtype, device=dev)
+        _lib.check(L.mlora_shrink(_lib.current_stream(dev), plan.handle, _lib.ptr(plan.scratch), plan.scratch.numel(),
+                                  _lib.ptr(wd.x[t.h_in]), w.T, t.h_in, R, pa, t.slot, 4, _lib.ptr(delta), R, 0, 0, 0, code))
+        torch.cuda.synchronize()
+        assert_parity(y.cpu(), want_y, f"one-launch op, round {rep}")
+        assert_parity(delta.cpu(), want_d, f"split-K shrink on the same plan, round {rep}")
+        if first is None:
+            first = (y.clone(), delta.clone())
+        assert torch.equal(y, first[0]) and torch.equal(delta, first[1])

@@ -127,7 +127,7 @@ void set_reduce_here(ShrinkArgs &a, const mlora_plan *plan, const PlanLayout &L,
   a.reduce_here = (small && a.ksplit > 1 && !a.partial_only) ? ((flags & MLORA_SHRINK_RECOMPUTE) ? 2 : 1) : 0;
   a.prp = (int)partial_stride_lines(max_rank);
   a.n_tiles = (int)tiles_upper(plan->T, plan->n_adapters, plan->bm_shrink);
-  a.arrive = reinterpret_cast<unsigned long long *>(static_cast<int32_t *>(plan->dev) + L.off_stamps);
+  a.arrive = reinterpret_cast<unsigned long long *>(static_cast<int32_t *>(plan->dev) + L.off_arrive);
 }
 
 struct Carver {

@@ -10,15 +10,16 @@ namespace mlora {
 
 // ---- plan buffer layout (int32 words) ------------------------------------------------------
 //   hdr[32] | perm[T] | padapter[T] | prank[T] | tiles_s[max_tiles][8] | tiles_e[max_tiles][8]
-//   | done[max_tiles] | stamps[max_tiles][DECODE_MAX_PRODUCERS] | scratch: cnt[A] gstart[A] toff_s[A] toff_e[A]
+//   | done[max_tiles] | stamps[max_tiles][DECODE_MAX_PRODUCERS] | arrive[max_tiles][2 * MLORA_MAX_TARGETS]
+//   | scratch: cnt[A] gstart[A] toff_s[A] toff_e[A]
 // perm[p]     token index at sorted position p (tokens grouped by adapter, original order kept
 //             inside a group); positions >= hdr[H_NACTIVE] are unused
 // padapter[p] adapter of position p;  prank[p] its rank
 // tile        {adapter, rank, first position, token count, a_start[adapter], 0, 0, 0}
 // done, stamps  the hand-off words of the one-launch op (csrc/decode.hip): per tile a count of the shrink items
-//             that have finished on this plan, and one stamp per shrink item; zeroed by the plan kernel.
-//             The stamps of tile t also serve as the arrival words of the shrink's own split-K sum
-//             (csrc/shrink.hip), 8 x 64 bits per tile, zero between launches
+//             that have finished on this plan, and one stamp per shrink item; zeroed by the plan kernel
+// arrive      the arrival words of the shrink's own split-K sum (csrc/shrink.hip): one 64-bit word per tile and
+//             target, zeroed by the plan kernel and back at zero after every launch
 constexpr int HDR_WORDS = 32;
 constexpr int TILE_WORDS = 8;
 constexpr int32_t PLAN_MAGIC = 0x4d4c5241;
@@ -36,7 +37,8 @@ constexpr int DECODE_MAX_PRODUCERS = 16;   // shrink items per tile (K chunks x 
 
 struct PlanLayout {
   int64_t T, A, max_tiles;
-  int64_t off_perm, off_padapter, off_prank, off_tiles_s, off_tiles_e, off_counters, off_stamps, off_scratch, total_words;
+  int64_t off_perm, off_padapter, off_prank, off_tiles_s, off_tiles_e, off_counters, off_stamps, off_arrive, off_scratch,
+      total_words;
 };
 
 static inline __host__ __device__ int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
@@ -53,7 +55,8 @@ static inline PlanLayout plan_layout(int64_t T, int64_t A) {
   L.off_tiles_e = L.off_tiles_s + L.max_tiles * TILE_WORDS;
   L.off_counters = L.off_tiles_e + L.max_tiles * TILE_WORDS;
   L.off_stamps = align_up(L.off_counters + L.max_tiles, 32);
-  L.off_scratch = align_up(L.off_stamps + L.max_tiles * DECODE_MAX_PRODUCERS, 8);
+  L.off_arrive = align_up(L.off_stamps + L.max_tiles * DECODE_MAX_PRODUCERS, 8);
+  L.off_scratch = align_up(L.off_arrive + L.max_tiles * 2 * MLORA_MAX_TARGETS, 8);
   L.total_words = L.off_scratch + 4 * A + 8;
   return L;
 }
@@ -105,7 +108,7 @@ struct ShrinkArgs {
   int reduce_here;            // 0 off, 1 on, 2 on with every sum taking the recompute path (tests)
   int prp;                    // row stride of the partials in that mode: whole 128-byte lines per row
   int n_tiles;                // upper bound of the tile count
-  unsigned long long *arrive; // [tiles][MLORA_MAX_TARGETS * 2] arrival words, zero between launches
+  unsigned long long *arrive; // [tiles][MLORA_MAX_TARGETS] arrival words, zero between launches
 };
 
 struct ExpandArgs {

@@ -175,7 +175,7 @@ __global__ __launch_bounds__(256) void shrink_kernel(const int32_t *tiles_base, 
   __syncthreads();
   if (tid == 0) {
     const uint32_t xcd = xcd_id();
-    unsigned long long *word = p.arrive + (int64_t)tile_idx * (2 * MLORA_MAX_TARGETS) + z_idx;
+    unsigned long long *word = p.arrive + (int64_t)tile_idx * MLORA_MAX_TARGETS + z_idx;
     const unsigned long long add = 1ull + (xcd < 8 ? 1ull << (8 + 7 * xcd) : 0ull);
     const unsigned long long now = __hip_atomic_fetch_add(word, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + add;
     int last = 0;
