@@ -40,11 +40,15 @@ def reference_layer(x, w, wl, seq_lens, heads, cos, sin, with_lora=True):
     return x + proj(m, w.w_down, "down")
 
 
-@pytest.mark.parametrize("n,kw", [(3, dict(hidden=256, mlp=704, len_div=8, n_decode=40)),
-                                  (5, dict(hidden=256, mlp=704, len_div=8, n_decode=48, n_adapters=20))])
-def test_layer_forward_with_lora_on_seven_projections(dev, n, kw):
+@pytest.mark.parametrize("n,kw,shape", [
+    (3, dict(hidden=256, mlp=704, len_div=8, n_decode=40), (256, 704, 8)),
+    (5, dict(hidden=256, mlp=704, len_div=8, n_decode=48, n_adapters=20), (256, 704, 8)),
+    # configuration 5 at its full size: 7B shape, 1152 tokens, 64 resident adapters of ranks 16-64
+    (5, dict(), (4096, 11008, 32)),
+], ids=["config3-small", "config5-small", "config5-full"])
+def test_layer_forward_with_lora_on_seven_projections(dev, n, kw, shape):
     wl = W.CONFIGS[n](targets=NAMES, **kw)
-    H, MLP, heads, dt = 256, 704, 8, wl.dtype
+    (H, MLP, heads), dt = shape, wl.dtype
     g = torch.Generator().manual_seed(100 + n)
     # LoRA weights large enough that dropping them is far outside the tolerance
     for name in ("q", "gate", "down"):
