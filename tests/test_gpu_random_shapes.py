@@ -141,3 +141,40 @@ def test_many_k_chunks(dev, bm_shrink, ksplit, h_in):
         plan.apply(y, x.to(dev), pd.key_buffer, pd.value_buffer, pd.a_start, pd.a_len, pd.a_loc, 2, pd.a_scaling)
         assert_parity(y.cpu(), want, f"ksplit {ksplit} h_in {h_in} bm {bm_shrink} rie {rie}")
         assert torch.equal(y.cpu()[ids < 0], y0[ids < 0])
+
+
+TABLE_CASES = [
+    # (hidden, tokens, rank, resident adapters): shapes of the widths the tile table holds measured entries
+    # for beside 4096 and 11008, decode-like and prefill-like, through the configuration the table gives them
+    (5120, 8, 16, 8), (5120, 64, 32, 32), (5120, 256, 16, 100), (5120, 1000, 64, 8), (5120, 2300, 128, 8),
+    (6144, 5, 64, 8), (6144, 64, 16, 32), (6144, 256, 32, 32), (6144, 700, 16, 100), (6144, 3000, 64, 32),
+    (8192, 8, 32, 8), (8192, 40, 128, 8), (8192, 256, 16, 8), (8192, 1024, 32, 32), (8192, 2048, 64, 8),
+    (13824, 3, 16, 8), (13824, 64, 64, 32), (13824, 200, 16, 32), (13824, 900, 32, 8), (13824, 2100, 64, 8),
+]
+
+
+@pytest.mark.parametrize("hidden,T,rank,n_adapters", TABLE_CASES)
+def test_table_configurations_of_other_widths(dev, hidden, T, rank, n_adapters):
+    """The plan takes its tile heights, split-K count and launch structure from the table entry of the shape
+    (one launch for several of the small ones); whatever the entry says, the result is the oracle's."""
+    from valora_amd import tile_table
+    g = torch.Generator().manual_seed(hidden + T + rank)
+    dtype = torch.bfloat16 if (T + rank) % 32 else torch.float16
+    h_out = 4096 if hidden > 8192 else hidden          # 13824 is an MLP width: down-projection shape
+    pool = W.make_pool([rank] * n_adapters, hidden, h_out, dtype, g, True, n_slots=1, std=0.03, heads=1)
+    req = 1 if T <= 1024 else 128
+    ids = torch.repeat_interleave(W.zipf_ids(n_adapters, (T + req - 1) // req, 0.7, g), req)[:T]
+    x = torch.randn(T, hidden, generator=g).to(dtype)
+    y0 = torch.randn(T, h_out, generator=g).to(dtype)
+    cfg = tile_table.lookup(T, rank, hidden, n_adapters)
+    what = f"hidden {hidden} T {T} rank {rank} adapters {n_adapters}: {cfg}"
+    print(what, flush=True)
+    pd = pool.to(dev)
+    plan = LoraPlan(ids.to(dev), pd.a_start, pd.a_len, rank, n_slots=1, hidden=hidden)
+    assert (plan.bm_shrink, plan.bm_expand) == ((16, 16) if plan.one_launch else (cfg.bm_shrink, cfg.bm_expand))
+    assert plan.one_launch == (cfg.one_launch and rank <= 64)
+    y = y0.to(dev)
+    plan.apply(y, x.to(dev), pd.key_buffer, pd.value_buffer, pd.a_start, pd.a_len, pd.a_loc, 0, pd.a_scaling)
+    want = O.lora_op(y0, x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, 0,
+                     pool.a_scaling, n_slots=1)
+    assert_parity(y.cpu(), want, what)
