@@ -147,3 +147,49 @@ def test_install_aliases_registers_the_reference_import_names():
             sys.modules.pop(n, None)
             if m is not None:
                 sys.modules[n] = m
+
+
+C_PROGRAM = r"""
+#include <stdio.h>
+#include <string.h>
+#include "mlora.h"
+int main(void) {
+  mlora_tile_config c;
+  mlora_plan plan;
+  memset(&plan, 0, sizeof plan);
+  if (mlora_version() <= 0) return 1;
+  if (mlora_plan_bytes(256, 64) == 0 || mlora_workspace_bytes(256, 64, 16) == 0) return 2;
+  if (mlora_tile_lookup(256, 16, 4096, 64, &c) != MLORA_OK || c.bm_shrink <= 0) return 3;
+  /* a call the library must refuse before it touches a device */
+  if (mlora_build_plan(NULL, &plan, NULL, 8, NULL, NULL, 0, 4, 16, 16) == MLORA_OK) return 4;
+  if (mlora_last_error() == NULL || strlen(mlora_last_error()) == 0) return 5;
+  printf("ok %d\n", mlora_version());
+  return 0;
+}
+"""
+
+
+def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
+    """include/mlora.h is the boundary a foreign-language binding is written against: it has to compile as
+    C99 and as C++ without warnings, and a C program has to link against libmlora.so and get answers from the
+    calls that need no GPU."""
+    import shutil
+    import subprocess
+    gcc, gxx = shutil.which("gcc"), shutil.which("g++")
+    if gcc is None or gxx is None:
+        pytest.skip("no host compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    inc = os.path.join(root, "include")
+    src = tmp_path / "use_mlora.c"
+    src.write_text(C_PROGRAM)
+    for cmd in ([gcc, "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-I", inc, str(src)],
+                [gxx, "-std=c++11", "-pedantic", "-Wall", "-Wextra", "-Werror", "-fsyntax-only", "-x", "c++", "-I", inc, str(src)]):
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr
+    exe = tmp_path / "use_mlora"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    r = subprocess.run([gcc, "-std=c99", "-I", inc, str(src), "-L", libdir, "-lmlora", f"-Wl,-rpath,{libdir}",
+                        "-Wl,-rpath,/opt/rocm/lib", "-o", str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0 and r.stdout.startswith("ok"), (r.returncode, r.stdout, r.stderr)
