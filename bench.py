@@ -457,6 +457,30 @@ def bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, r
     out["layer_us_is"] = "q+k+v in one mlora_lora_apply_multi call + o in one mlora_lora_apply call, per layer"
     del yk, yv, yo
 
+    # -- the op between its producer and its consumer: y = x @ W (the base projection) -> the op on y -> a kernel
+    #    that reads y, per layer with distinct weights; the difference to the same loop without the op is what the op
+    #    costs where y is warm from the projection and wanted again right after
+    gw = torch.Generator(device=dev).manual_seed(2004)
+    Ws = [(torch.randn(H, H, generator=gw, device=dev) * 0.02).to(w.dtype) for _ in range(L)]
+    zs = [torch.empty(T, H, dtype=w.dtype, device=dev) for _ in range(L)]
+
+    def forward(lora):
+        def run():
+            for l in range(L):
+                torch.mm(xs[l], Ws[l], out=ys[l])
+                if lora:
+                    plan.apply(ys[l], xs[l], kb[l], vb[l], *idx, 0, p.a_scaling)
+                torch.mul(ys[l], 0.5, out=zs[l])
+        return run
+
+    ms_base, _ = time_graph(torch, forward(False), reps, 5, use_graph)
+    ms_lora, _ = time_graph(torch, forward(True), reps, 5, use_graph)
+    out["in_forward"] = {"base_us_per_layer": round(ms_base * 1e3 / L, 3), "with_lora_us_per_layer": round(ms_lora * 1e3 / L, 3),
+                         "lora_us_per_layer": round((ms_lora - ms_base) * 1e3 / L, 3),
+                         "is": "per layer: y = x @ W (torch.mm) -> the LoRA op on y -> an elementwise kernel that reads y; "
+                               "the op's cost = difference to the same loop without it"}
+    del Ws, zs
+
     # -- the reference's entry points: delta = shrink(x); y += expand(delta), two calls per layer
     delta = [torch.zeros(T, R, dtype=w.dtype, device=dev) for _ in range(L)]
 
