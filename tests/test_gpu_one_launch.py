@@ -243,3 +243,35 @@ def test_one_launch_op_and_in_launch_split_k_sum_share_a_plan(dev):
         if first is None:
             first = (y.clone(), delta.clone())
         assert torch.equal(y, first[0]) and torch.equal(delta, first[1])
+
+
+def test_two_streams_with_a_plan_each_run_side_by_side(dev):
+    """Two layer loops on two streams, each with its own plan, scratch and outputs, overlap on the device: neither
+    grid has the device to itself, so items start late and waits run out -- every wait is bounded and the give-up
+    path gives the same bits, so both loops finish and equal their serial two-launch results."""
+    L = 12
+    sides = []
+    for k, (n_tokens, n_adapters) in enumerate(((256, 64), (200, 48))):
+        w = W.config2(hidden=2048, n_tokens=n_tokens, n_adapters=n_adapters)
+        wd = w.to(dev)
+        p = wd.target("q").pool
+        one, two = _pair(wd, "q", max(p.ranks), 2048, 4)
+        g = torch.Generator(device=dev).manual_seed(40 + k)
+        xs = [torch.randn(w.T, 2048, generator=g, device=dev).to(w.dtype) for _ in range(L)]
+        y0 = [torch.randn(w.T, 2048, generator=g, device=dev).to(w.dtype) for _ in range(L)]
+        want = [y.clone() for y in y0]
+        for l in range(L):
+            two.apply(want[l], xs[l], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, l % 4, p.a_scaling)
+        sides.append((one, p, xs, y0, want, torch.cuda.Stream(device=dev)))
+    torch.cuda.synchronize()
+    for rep in range(3):
+        outs = [[y.clone() for y in side[3]] for side in sides]
+        torch.cuda.synchronize()
+        for l in range(L):                      # enqueue alternately so that the two streams' launches overlap
+            for (one, p, xs, _, _, s), out in zip(sides, outs):
+                with torch.cuda.stream(s):
+                    one.apply(out[l], xs[l], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, l % 4, p.a_scaling)
+        torch.cuda.synchronize()
+        for k, (side, out) in enumerate(zip(sides, outs)):
+            for l in range(L):
+                assert torch.equal(out[l], side[4][l]), f"repetition {rep}, stream {k}, layer {l}"
