@@ -105,3 +105,27 @@ def test_rows_beyond_two_to_the_31_elements(dev):
     want = O.lora_op(y0_s, x_s, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids_s, 0,
                      pool.a_scaling, n_slots=1)
     assert_parity(y[rows.to(dev)].cpu(), want, "rows at both ends of a 2**31-element matrix")
+
+
+def test_row_scatter_and_gather_in_a_pool_beyond_4_gib(dev):
+    """A pool of 8 layers x 70 000 rows x 4096 fp16 (4.6 GB, more than 2**31 elements): rows near the end of the last
+    layers are written and read back; torch's indexed assignment on the same tensor is the checker
+    (valora/server/router/model_infer/infer_adapter.py:59 is exactly that assignment)."""
+    layers, rows, H, n = 8, 70_000, 4096, 192
+    assert layers * rows * H > (1 << 31)
+    g = torch.Generator(device=dev).manual_seed(5)
+    pool = torch.zeros(layers, rows, H, dtype=torch.float16, device=dev)
+    packed = torch.randn(layers, n, H, generator=g, device=dev, dtype=torch.float32).half()
+    loc = torch.cat([torch.arange(rows - n // 2, rows), torch.randperm(rows - n, generator=torch.Generator().manual_seed(6))[:n // 2]])
+    loc_d = loc.to(dev)
+    st = _lib.current_stream(dev)
+    esz = 2
+    _lib.check(_lib.lib().mlora_pool_scatter_rows(st, _lib.ptr(pool), rows, rows * H * esz, _lib.ptr(packed),
+                                                  n * H * esz, _lib.ptr(loc_d), n, H * esz, layers))
+    for l in (0, layers - 1):
+        assert torch.equal(pool[l][loc_d], packed[l])
+    assert int(pool.count_nonzero()) == int(packed.count_nonzero())      # nothing written anywhere else
+    back = torch.empty_like(packed)
+    _lib.check(_lib.lib().mlora_pool_gather_rows(st, _lib.ptr(pool), rows, rows * H * esz, _lib.ptr(back),
+                                                 n * H * esz, _lib.ptr(loc_d), n, H * esz, layers))
+    assert torch.equal(back, packed)
