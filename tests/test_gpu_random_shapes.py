@@ -150,17 +150,20 @@ TABLE_CASES = [
     (6144, 5, 64, 8), (6144, 64, 16, 32), (6144, 256, 32, 32), (6144, 700, 16, 100), (6144, 3000, 64, 32),
     (8192, 8, 32, 8), (8192, 40, 128, 8), (8192, 256, 16, 8), (8192, 1024, 32, 32), (8192, 2048, 64, 8),
     (13824, 3, 16, 8), (13824, 64, 64, 32), (13824, 200, 16, 32), (13824, 900, 32, 8), (13824, 2100, 64, 8),
+    (2048, 8, 16, 8), (2048, 256, 32, 32), (2048, 3000, 64, 8), (3072, 60, 64, 8), (3072, 1024, 16, 100),
+    (7168, 7, 32, 8), (7168, 256, 16, 32), (7168, 2500, 128, 8), (14336, 64, 16, 32), (14336, 1500, 64, 8),
+    (28672, 8, 16, 8), (28672, 200, 32, 8), (28672, 1100, 64, 8),
 ]
 
 
 @pytest.mark.parametrize("hidden,T,rank,n_adapters", TABLE_CASES)
 def test_table_configurations_of_other_widths(dev, hidden, T, rank, n_adapters):
-    """The plan takes its tile heights, split-K count and launch structure from the table entry of the shape
+    """Widths 2048 ... 28672.  The plan takes its tile heights, split-K count and launch structure from the table entry of the shape
     (one launch for several of the small ones); whatever the entry says, the result is the oracle's."""
     from valora_amd import tile_table
     g = torch.Generator().manual_seed(hidden + T + rank)
     dtype = torch.bfloat16 if (T + rank) % 32 else torch.float16
-    h_out = 4096 if hidden > 8192 else hidden          # 13824 is an MLP width: down-projection shape
+    h_out = 4096 if hidden > 8192 else hidden          # 13824 and wider are MLP widths: down-projection shape
     pool = W.make_pool([rank] * n_adapters, hidden, h_out, dtype, g, True, n_slots=1, std=0.03, heads=1)
     req = 1 if T <= 1024 else 128
     ids = torch.repeat_interleave(W.zipf_ids(n_adapters, (T + req - 1) // req, 0.7, g), req)[:T]

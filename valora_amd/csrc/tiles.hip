@@ -73,8 +73,34 @@ mlora_tile_config tile_fallback(int64_t T, int64_t max_rank, int64_t hidden, int
   return c;
 }
 
+static bool table_lookup(int64_t max_rank, int64_t hidden, int64_t tb, int64_t rb, int64_t ab, mlora_tile_config &c);
+
+// The table is scanned linearly; a serving loop asks for the same few shapes call after call, so each thread
+// remembers its last answers.  (T and the rank enter the answer beyond their buckets only through max_rank > 64,
+// which the rank bucket already tells.)
 mlora_tile_config tile_lookup(int64_t T, int64_t max_rank, int64_t hidden, int64_t A) {
   const int64_t tb = bucket(T, kTokenBuckets), rb = bucket(max_rank, kRankBuckets), ab = bucket(A, kAdapterBuckets);
+  struct Memo {
+    int64_t tb, rb, hidden, ab;
+    mlora_tile_config cfg;
+    bool valid;
+  };
+  constexpr int N_MEMO = 8;
+  static thread_local Memo memo[N_MEMO];
+  static thread_local int next = 0;
+  for (int i = 0; i < N_MEMO; ++i)
+    if (memo[i].valid && memo[i].tb == tb && memo[i].rb == rb && memo[i].hidden == hidden && memo[i].ab == ab)
+      return memo[i].cfg;
+  mlora_tile_config c;
+  // the rule for shapes without an entry looks at T and A themselves, not at their buckets: not remembered
+  if (!table_lookup(max_rank, hidden, tb, rb, ab, c)) return tile_fallback(T, max_rank, hidden, A);
+  memo[next] = Memo{tb, rb, hidden, ab, c, true};
+  next = (next + 1) % N_MEMO;
+  return c;
+}
+
+// the entry of the shape's buckets (of the nearest measured width, if this one has none); false: no entry
+static bool table_lookup(int64_t max_rank, int64_t hidden, int64_t tb, int64_t rb, int64_t ab, mlora_tile_config &c) {
   const Entry *e = find(tb, rb, hidden, ab);
   bool other_width = false;
   if (!e) {
@@ -91,8 +117,8 @@ mlora_tile_config tile_lookup(int64_t T, int64_t max_rank, int64_t hidden, int64
     }
     other_width = e != nullptr;
   }
-  if (!e) return tile_fallback(T, max_rank, hidden, A);
-  mlora_tile_config c{e->bm_shrink, e->ksplit, e->bm_expand, e->flags};
+  if (!e) return false;
+  c = mlora_tile_config{e->bm_shrink, e->ksplit, e->bm_expand, e->flags};
   if (other_width) {   // the split-K factor cut to what the width can be split into
     const int64_t kcap = hidden / 128 > 1 ? hidden / 128 : 1;
     if (c.ksplit > kcap) c.ksplit = (int32_t)kcap;
@@ -104,7 +130,7 @@ mlora_tile_config tile_lookup(int64_t T, int64_t max_rank, int64_t hidden, int64
     c.flags &= ~MLORA_ONE_LAUNCH;
   }
   if (c.flags & MLORA_ONE_LAUNCH) c.flags |= MLORA_REDUCE_IN_EXPAND;
-  return c;
+  return true;
 }
 
 // split-K factor for a plan that was cut with shrink tiles of `bm` tokens: the table's, if its entry for this
