@@ -94,7 +94,7 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
   constexpr int N_WAVES = THREADS / 64;
   __shared__ int32_t whist[HIST_WORDS];
   __shared__ Quad wsum[PLAN_WAVES + 1];
-  __shared__ int s_maxrank;
+  __shared__ int s_wmaxr[PLAN_WAVES];
   __shared__ int s_err;
 
   __shared__ int32_t s_tab[SMALL ? 4 * PLAN_SMALL_A : 1];
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
       s_astart[a] = a == tid ? start0 : a_start[a];
     }
   }
-  if (tid == 0) { s_maxrank = 0; s_err = 0; }
+  if (tid == 0) s_err = 0;
   __syncthreads();
   for (int i = tid; i < n_flag_words; i += THREADS) plan[off_counters + i] = 0;
 
@@ -176,7 +176,14 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
   const Quad pre = block_exclusive_scan4(Quad{my_c, my_ts, my_te, my_g}, &tot, wsum, N_WAVES);
   const int n_active = tot.c, n_ts = tot.ts, n_te = tot.te, n_g = tot.g;
   int pre_c = pre.c, pre_ts = pre.ts, pre_te = pre.te;
-  if (my_maxr > 0) atomicMax(&s_maxrank, my_maxr);
+  {
+    // widest rank among the adapters that have tokens.  Ranks are multiples of 8 up to MAX_RANK: a few votes per wave
+    // find the wave's maximum (an LDS atomic per lane is serialised lane by lane by the compiler: 1.8 us here)
+    int wave_maxr = 0;
+    for (int rr = MAX_RANK; rr >= 8; rr -= 8)
+      if (__ballot(my_maxr >= rr)) { wave_maxr = rr; break; }
+    if (lane == 0) s_wmaxr[wave] = wave_maxr;
+  }
   for (int a = a_beg; a < a_endx; ++a) {
     const int c = cnt[a];
     gstart[a] = pre_c;
@@ -196,6 +203,7 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
 
   // 3. stable scatter: each wave walks its range in order, 64 tokens a step; lanes holding the
   //    same adapter get consecutive positions in lane order.
+  const int a_bits = A > 1 ? 32 - __clz(A - 1) : 0;   // bits that tell two adapter indices apart
   for (int t0 = t_beg; t0 < t_end; t0 += 64) {
     const int t = t0 + lane;
     int a = -1, r = 0;
@@ -209,45 +217,25 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
         if (r > 0) a = (int)a64;
       }
     }
-    // Lanes holding the same adapter get consecutive positions in lane order.  A prefill batch has one or two
-    // adapters per 64 tokens: a few rounds of "take the first unplaced lane's adapter and place all its lanes"
-    // finish the step.  A decode batch has almost as many adapters as tokens, and a round costs an LDS round
-    // trip: what is left after four rounds is placed by rank instead (lanes before me with my adapter, found
-    // with 64 uniform-lane reads).
-    unsigned long long remaining = __ballot(a >= 0);
-    for (int round = 0; remaining && round < 4; ++round) {
-      const int leader = __ffsll((long long)remaining) - 1;
-      const int a0 = __shfl(a, leader, 64);
-      const unsigned long long m = __ballot(a == a0);
-      const int slot_idx = wave * A + a0;
-      const int base = whist[slot_idx];
-      if (a == a0) {
-        const int pos = base + __popcll(m & ((1ull << lane) - 1ull));
-        perm[pos] = t;
-        padapter[pos] = a0;
-        prank[pos] = r;
+    // Lanes holding the same adapter get consecutive positions in lane order.  Which lanes hold my adapter comes from
+    // one vote per bit of the adapter index (6 votes for 64 adapters), whatever the mix: one adapter for all 64 tokens
+    // of a prefill request or 64 different ones in a decode batch.
+    const unsigned long long valid = __ballot(a >= 0);
+    if (valid) {   // wave-uniform
+      unsigned long long same = valid;
+      for (int b = 0; b < a_bits; ++b) {
+        const bool bit = (a >> b) & 1;
+        const unsigned long long m = __ballot(bit);
+        same &= bit ? m : ~m;
       }
-      __builtin_amdgcn_wave_barrier();
-      if (lane == leader) whist[slot_idx] = base + __popcll(m);
-      __builtin_amdgcn_wave_barrier();
-      remaining &= ~m;
-    }
-    if (remaining) {   // wave-uniform
-      const bool mine = (remaining >> lane) & 1ull;
-      int before = 0, after = 0;
-      for (int d = 0; d < 64; ++d) {
-        const int other = __builtin_amdgcn_readlane(a, d);
-        before += (other == a && d < lane) ? 1 : 0;
-        after += (other == a && d > lane) ? 1 : 0;
-      }
-      if (mine) {
+      if (a >= 0) {
         const int slot_idx = wave * A + a;
-        const int pos = whist[slot_idx] + before;
+        const int pos = whist[slot_idx] + __popcll(same & ((1ull << lane) - 1ull));
         perm[pos] = t;
         padapter[pos] = a;
         prank[pos] = r;
-        __builtin_amdgcn_wave_barrier();            // every lane of the group has read the offset ...
-        if (after == 0) whist[slot_idx] = pos + 1;  // ... before its last lane moves it on
+        __builtin_amdgcn_wave_barrier();                           // every lane of the group has read the offset ...
+        if (((same >> lane) >> 1) == 0) whist[slot_idx] = pos + 1;   // ... before its last lane moves it on
       }
       __builtin_amdgcn_wave_barrier();
     }
@@ -255,7 +243,8 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
   __syncthreads();
 
   // 4. tile lists: tile i belongs to the last adapter whose tile offset is <= i
-  for (int pass = 0; pass < 2; ++pass) {
+  const bool one_list = bm_s == bm_e;   // then both lists are the same records (the one-launch op: 16 / 16)
+  for (int pass = 0; pass < (one_list ? 1 : 2); ++pass) {
     const int n_tiles = pass ? n_te : n_ts;
     const int bm = pass ? bm_e : bm_s;
     const int32_t *toff = pass ? toff_e : toff_s;
@@ -272,21 +261,23 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
       const int64_t st = start_of(a);
       const bool st_bad = st < 0 || st > 0x7fffffff;
       if (st_bad) atomicOr(&s_err, (int)PERR_START_OVERFLOW);
-      int32_t *tl = tiles + (int64_t)i * TILE_WORDS;
-      tl[0] = a;
-      tl[1] = rank_of(a);
-      tl[2] = gstart[a] + k * bm;
-      tl[3] = min(bm, c - k * bm);
-      tl[4] = st_bad ? INT32_MIN / 2 : (int32_t)st;   // an index position no look-up accepts
-      tl[5] = 0; tl[6] = 0; tl[7] = 0;
+      const int32_t rec[5] = {a, rank_of(a), gstart[a] + k * bm, min(bm, c - k * bm),
+                              st_bad ? INT32_MIN / 2 : (int32_t)st};   // an index position no look-up accepts
+      for (int list = 0; list < (one_list ? 2 : 1); ++list) {
+        int32_t *tl = (list ? plan + off_tiles_e : tiles) + (int64_t)i * TILE_WORDS;
+#pragma unroll
+        for (int q = 0; q < TILE_WORDS; ++q) tl[q] = q < 5 ? rec[q] : 0;
+      }
     }
     // the kernels' grids are sized with the upper bound of the tile count: records past the last
     // tile say "no tokens", so a workgroup needs no second look-up to know that it has nothing to do
     const int upper = (T + bm - 1) / bm + min(A, T);
     for (int i = n_tiles + tid; i < upper; i += THREADS) {
-      int32_t *tl = tiles + (int64_t)i * TILE_WORDS;
+      for (int list = 0; list < (one_list ? 2 : 1); ++list) {
+        int32_t *tl = (list ? plan + off_tiles_e : tiles) + (int64_t)i * TILE_WORDS;
 #pragma unroll
-      for (int k = 0; k < TILE_WORDS; ++k) tl[k] = 0;
+        for (int k = 0; k < TILE_WORDS; ++k) tl[k] = 0;
+      }
     }
   }
   __syncthreads();
@@ -297,7 +288,9 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
     plan[H_NTILES_S] = n_ts;
     plan[H_NTILES_E] = n_te;
     plan[H_NGROUPS] = n_g;
-    plan[H_MAXRANK] = s_maxrank;
+    int maxrank = 0;
+    for (int wv = 0; wv < N_WAVES; ++wv) maxrank = max(maxrank, s_wmaxr[wv]);
+    plan[H_MAXRANK] = maxrank;
     plan[H_ERR] = s_err;
     plan[H_BM_S] = bm_s;
     plan[H_BM_E] = bm_e;
