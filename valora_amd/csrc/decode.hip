@@ -132,29 +132,57 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
   const bool on_time = id < h_resident;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int rp = a.s.rp;
-  const int32_t *__restrict__ perm = a.s.plan + a.s.off_perm;
 
   const ItemId it = item_of(h_n_producers, h_n_consumers, h_groups_per_chunk, id);
   const bool shrink_item = it.shrink;
   const int item = it.item, tile_idx = it.tile;
   if (tile_idx >= h_n_tiles) return;
-  const int32_t *__restrict__ tile = tiles_base + (int64_t)tile_idx * TILE_WORDS;
-  const int ad = tile[0], r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
-  if (cnt <= 0) return;   // records past the last tile are zero
   if (shrink_item && !on_time) return;
-  // the launch's tag: what the tile's `done` word holds while none of this launch's shrink items has finished
-  const uint32_t want_stamp = stamp_of(done_base[tile_idx], xcd_id());
-  uint32_t *const stamps = a.stamps + (int64_t)tile_idx * DECODE_MAX_PRODUCERS;
-  // a tile's partials: [target][K chunk][16 rows][rp] floats, whole lines of the tile's own
-  float *const tile_partial = a.s.partial + (int64_t)tile_idx * a.n_producers * 16 * rp;
+  const int32_t *__restrict__ tile = tiles_base + (int64_t)tile_idx * TILE_WORDS;
+
+  // ONE scalar round trip per shrink item before its vector loads: the tile record, the tile's `done` word and every
+  // field of the argument block the item is going to use are requested together and waited for once.  Left to
+  // itself the compiler fetches each group of argument fields right before its first use, behind the previous
+  // wait -- seven dependent scalar round trips in front of the first operand load, each an L2 access while all
+  // workgroups of the grid start at the same moment.  The empty asm takes the values as read-write operands: they
+  // have to be in registers at that point, and cannot be fetched again later instead of being kept.
+  int ad = tile[0], r = tile[1], pos0 = tile[2], cnt = tile[3], astart = tile[4];
+  uint32_t done0 = done_base[tile_idx];
+  int rp = a.s.rp, n_producers = a.n_producers;
+  const int32_t *plan_words = a.s.plan;
+  int64_t off_perm = a.s.off_perm;
+  float *partial_base = a.s.partial;
+  uint32_t *stamps_base = a.stamps;
 
   // ------------------------------------------------------------------ shrink item
   if (shrink_item) {
-    const int z = item / a.s.ksplit, s = item - z * a.s.ksplit;
-    const int kbeg = s * a.s.kchunk;
-    const int kend = min(a.s.h_in, kbeg + a.s.kchunk);
-    shrink_tile_to_lds<T, 1, NB>(a.s.x, a.s.h_in, a.s.pool, a.s.slots[z], perm, r, pos0, cnt, astart, kbeg, kend, red);
+    const uint16_t *x = a.s.x;
+    PoolDev pool = a.s.pool;
+    int h_in = a.s.h_in, ksplit = a.s.ksplit, kchunk = a.s.kchunk;
+    int sl0 = a.s.slots[0], sl1 = a.s.slots[1], sl2 = a.s.slots[2], sl3 = a.s.slots[3];
+    uint32_t *done = a.done;
+    asm volatile("" : "+s"(ad), "+s"(r), "+s"(pos0), "+s"(cnt), "+s"(astart), "+s"(done0), "+s"(rp), "+s"(n_producers),
+                      "+s"(plan_words), "+s"(off_perm), "+s"(partial_base), "+s"(stamps_base), "+s"(x), "+s"(pool.w),
+                      "+s"(pool.w_rows), "+s"(pool.a_loc), "+s"(pool.a_loc_len), "+s"(h_in), "+s"(ksplit), "+s"(kchunk),
+                      "+s"(sl0), "+s"(sl1), "+s"(sl2), "+s"(sl3), "+s"(done));
+    if (cnt <= 0) return;   // records past the last tile are zero
+    x = as_global(x);
+    pool.w = as_global(pool.w);
+    pool.a_loc = as_global(pool.a_loc);
+    done = as_global(done);
+    partial_base = as_global(partial_base);
+    stamps_base = as_global(stamps_base);
+    const int32_t *__restrict__ perm = as_global(plan_words) + off_perm;
+    // the launch's tag: what the tile's `done` word holds while none of this launch's shrink items has finished
+    const uint32_t want_stamp = stamp_of(done0, xcd_id());
+    uint32_t *const stamps = stamps_base + (int64_t)tile_idx * DECODE_MAX_PRODUCERS;
+    // a tile's partials: [target][K chunk][16 rows][rp] floats, whole lines of the tile's own
+    float *const tile_partial = partial_base + (int64_t)tile_idx * n_producers * 16 * rp;
+    const int z = item / ksplit, s = item - z * ksplit;
+    const int kbeg = s * kchunk;
+    const int kend = min(h_in, kbeg + kchunk);
+    const int slot = z == 0 ? sl0 : z == 1 ? sl1 : z == 2 ? sl2 : sl3;
+    shrink_tile_to_lds<T, 1, NB>(x, h_in, pool, slot, perm, r, pos0, cnt, astart, kbeg, kend, red);
     if (wave == 0) {
       // wave 0 alone writes the partial and then the stamp: no barrier, and nothing else of its own in flight
       f32x4 *part = reinterpret_cast<f32x4 *>(tile_partial + (int64_t)item * 16 * rp);
@@ -168,19 +196,29 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
       wait_vmcnt<0>();
       if (lane == 0) __hip_atomic_store(stamps + item, want_stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     } else if (tid == 64) {
-      add_device(a.done + tile_idx, 1u);
+      add_device(done + tile_idx, 1u);
     }
     return;
   }
 
   // ------------------------------------------------------------------ expand item
-  const int z = item / a.e.n_ochunks, oc = item - z * a.e.n_ochunks;
-  const int rk = min(r, a.e.kmax);   // rank columns the narrow operand really has (bgmv_impl.cuh:167,186)
+  const int n_ochunks = a.e.n_ochunks, kmax = a.e.kmax, h_out = a.e.h_out, e_ksplit = a.e.ksplit, spin_limit = a.spin_limit;
+  const uint16_t *const scales = a.e.scales;
+  const int64_t *const a_loc = a.e.pool.a_loc;
+  const int64_t a_loc_len = a.e.pool.a_loc_len;
+  // (no joint round trip here: the expand items' loads are not what the op waits for -- requesting their argument
+  // fields early as well measured 0.04 us slower, the target's operands on top of that another 0.08 us)
+  if (cnt <= 0) return;   // records past the last tile are zero
+  const int32_t *__restrict__ perm = plan_words + off_perm;
+  const uint32_t want_stamp = stamp_of(done0, xcd_id());
+  uint32_t *const stamps = stamps_base + (int64_t)tile_idx * DECODE_MAX_PRODUCERS;
+  float *const tile_partial = partial_base + (int64_t)tile_idx * n_producers * 16 * rp;
+  const int z = item / n_ochunks, oc = item - z * n_ochunks;
+  const int rk = min(r, kmax);   // rank columns the narrow operand really has (bgmv_impl.cuh:167,186)
   const int slot = a.e.slots[z];
   uint16_t *const y = a.e.ys[z];
   const uint16_t *const wB = a.e.ws[z];
   const int64_t wB_rows = a.e.w_rows_t[z];
-  const int h_out = a.e.h_out;
 
   const int lrow = lane & 15, kg = lane >> 4;
   int o_wave[DEC_CH];
@@ -193,9 +231,9 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
   // array instead of being skipped, and their result is dropped.
   int my_perm = 0;
   if (tid < cnt) my_perm = perm[pos0 + tid];
-  const float scale = Tr::to_float(a.e.scales[ad]);
+  const float scale = Tr::to_float(scales[ad]);
   const float inv_h_out = 1.0f / (float)h_out;
-  const uint32_t base32 = (uint32_t)(astart + r * slot), n_loc = (uint32_t)a.e.pool.a_loc_len;
+  const uint32_t base32 = (uint32_t)(astart + r * slot), n_loc = (uint32_t)a_loc_len;
   const uint32_t step16 = 16u * (uint32_t)r;
   const bool can_step = step16 < (uint32_t)h_out;     // workgroup-uniform
   int64_t brow[DEC_CH][4][KB];
@@ -216,7 +254,7 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
         }
         const uint32_t idx = base32 + cur.bin;
         const bool ok = o < h_out && (int)j0 < rk && idx < n_loc;
-        brow[c][nb][kb] = a.e.pool.a_loc[ok ? idx : 0u];
+        brow[c][nb][kb] = a_loc[ok ? idx : 0u];
         boff[c][nb][kb] = cur.off;
         bok[c][nb][kb] = ok;
       }
@@ -254,8 +292,8 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
   //      verdict without draining its loads)
   if (wave == 0) {
     int ok = 0;
-    for (int it = 0; on_time && it < a.spin_limit; ++it) {
-      if (stamps_match(stamps, a.n_producers, want_stamp)) { ok = 1; break; }
+    for (int it = 0; on_time && it < spin_limit; ++it) {
+      if (stamps_match(stamps, n_producers, want_stamp)) { ok = 1; break; }
       __builtin_amdgcn_s_sleep(2);
     }
     if (lane == 0) s_ready = ok;
@@ -267,7 +305,7 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
   u32x4 vfrag[KB];
   const bool pok = lrow < cnt;
   if (ready) {
-    const float *part = tile_partial + (int64_t)z * a.e.ksplit * 16 * rp;
+    const float *part = tile_partial + (int64_t)z * e_ksplit * 16 * rp;
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
       const int j0 = kb * 32 + kg * 8;
@@ -275,11 +313,11 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
       if (pok && j0 < rk) {
         float f[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         const float *src0 = part + lrow * rp + j0;
-        for (int s0 = 0; s0 < a.e.ksplit; s0 += 4) {
+        for (int s0 = 0; s0 < e_ksplit; s0 += 4) {
           f32x4 lo[4], hi[4];
 #pragma unroll
           for (int u = 0; u < 4; ++u) {
-            const bool ok = s0 + u < a.e.ksplit;
+            const bool ok = s0 + u < e_ksplit;
             const f32x4 *src = reinterpret_cast<const f32x4 *>(src0 + (int64_t)(s0 + u) * 16 * rp);
             lo[u] = ok ? src[0] : f32x4{0.f, 0.f, 0.f, 0.f};
             hi[u] = ok ? src[1] : f32x4{0.f, 0.f, 0.f, 0.f};

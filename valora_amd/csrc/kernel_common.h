@@ -25,6 +25,13 @@ __device__ __forceinline__ void store16(uint16_t *p, u32x4 v) { *reinterpret_cas
 // Direct global -> LDS load: each active lane copies 16 bytes from its own global address to
 // lds_base + lane*16 (lds_base is wave-uniform); completion is tracked by vmcnt.
 #define GLOBAL_PTR(p) (reinterpret_cast<const __attribute__((address_space(1))) void *>(reinterpret_cast<uintptr_t>(p)))
+// A pointer that went through an inline asm operand has lost what the compiler knew about it; telling it again that
+// the memory is global keeps its loads and stores on the global path (flat accesses count against two wait counters)
+template <typename P>
+__device__ __forceinline__ P *as_global(P *p) {
+  typedef __attribute__((address_space(1))) P *GP;
+  return (P *)(GP)(uintptr_t)p;
+}
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
 // wait until at most N vector-memory loads of this wave are outstanding (loads retire in order)
