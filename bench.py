@@ -239,24 +239,28 @@ def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0, only_tar
     if not only:
         report["adapter_residency"] = bench_adapter_residency(torch, dev)
         report["config5_step"] = bench_config5_step(torch, W, dev, use_graph)
+        report["decode_step"] = bench_config5_step(torch, W, dev, use_graph, decode_only=True)
         report["config4_prefill_step"] = bench_config4_prefill_step(torch, W, dev, use_graph)
     with open(path, "w") as f:
         json.dump(report, f, indent=1)
 
 
-def bench_config5_step(torch, W, dev, use_graph):
+def bench_config5_step(torch, W, dev, use_graph, decode_only=False):
     """The serving step of benchmark configuration 5: 32 decoder layers of the 7B shape (hidden 4096, 32 heads,
     MLP 11008, random weights), 128 decode tokens with cached contexts of 256..2048 tokens plus 2 prefill
     requests of 512 tokens, 64 resident adapters (ranks 16/32/64, Zipf 0.8), LoRA on all 7 projections.  The base
     model is stock PyTorch (mm, scaled_dot_product_attention); reported: step time with LoRA, base-only step time
-    and their difference.  The KV cache is shared by the layers (it only serves the timing of the base step)."""
+    and their difference.  The KV cache is shared by the layers (it only serves the timing of the base step).
+    ``decode_only``: the same step for the decode batch of configuration 2 instead (256 tokens, one per request,
+    64 adapters of rank 16, fp16, no prefill requests)."""
     import torch.nn.functional as F
     from valora_amd.layer import LayerPlans, LayerPools, LayerWeights, layer_forward
-    H, MLP, heads, L, dt = 4096, 11008, 32, 32, torch.bfloat16
+    H, MLP, heads, L = 4096, 11008, 32, 32
     d = H // heads
-    w5 = W.CONFIGS[5]()
+    w5 = W.decode_layer() if decode_only else W.CONFIGS[5]()
+    dt = w5.dtype
     wd = w5.to(dev)
-    T, n_dec = w5.T, 128
+    T, n_dec = w5.T, (w5.T if decode_only else 128)
     pa, pu, pdn = wd.target("q").pool, wd.target("gate").pool, wd.target("down").pool
     idx = (pa.a_start, pa.a_len, pa.a_loc, pa.a_scaling)
     g = torch.Generator(device=dev).manual_seed(55)
@@ -272,11 +276,13 @@ def bench_config5_step(torch, W, dev, use_graph):
         layers.append((wts, pools))
     plans = LayerPlans(wd.ids, pa.a_start, pa.a_len, max(pa.ranks), H, MLP)
     gl = torch.Generator().manual_seed(56)
-    kv_len = torch.randint(256, 2049, (n_dec,), generator=gl)
+    # (decode only: short contexts, so that stock PyTorch's masked attention does not bury the difference the
+    # step is run for under its own run-to-run spread)
+    kv_len = torch.randint(64, 257, (n_dec,), generator=gl) if decode_only else torch.randint(256, 2049, (n_dec,), generator=gl)
     Lmax = int(kv_len.max())
     kc, vc = rnd(n_dec, heads, Lmax, d), rnd(n_dec, heads, Lmax, d)
     mask = (torch.arange(Lmax)[None, :] < kv_len[:, None]).to(dev)[:, None, None, :]
-    pre = [(n_dec + i * 512, n_dec + (i + 1) * 512) for i in range(2)]
+    pre = [] if decode_only else [(n_dec + i * 512, n_dec + (i + 1) * 512) for i in range(2)]
 
     def attention(q, k, v):
         out = torch.empty_like(q)
@@ -287,7 +293,7 @@ def bench_config5_step(torch, W, dev, use_graph):
             out[b:e] = F.scaled_dot_product_attention(qq, kk, vv, is_causal=True)[0].transpose(0, 1).reshape(512, H)
         return out
 
-    pos = torch.cat((kv_len.float(), torch.arange(512).float(), torch.arange(512).float())).to(dev)
+    pos = torch.cat([kv_len.float()] + [torch.arange(512).float() for _ in pre]).to(dev)
     freq = 1.0 / (10000 ** (torch.arange(0, d, 2, device=dev).float() / d))
     ang = torch.cat((pos[:, None] * freq[None], pos[:, None] * freq[None]), dim=-1)
     cos, sin = ang.cos().to(dt), ang.sin().to(dt)
@@ -300,13 +306,14 @@ def bench_config5_step(torch, W, dev, use_graph):
         return x
 
     out = {}
+    reps = 20 if decode_only else 5
     for name, lora in (("base_only", False), ("with_lora", True)):
         try:
-            ms, _ = time_graph(torch, lambda: step(lora), 5, 2, use_graph)
+            ms, _ = time_graph(torch, lambda: step(lora), reps, 2, use_graph)
             mode = "hip graph replay" if use_graph else "eager"
         except Exception as exc:   # a library call that cannot be captured: time it eagerly
             torch.cuda.synchronize()
-            ms, _ = time_graph(torch, lambda: step(lora), 5, 2, False)
+            ms, _ = time_graph(torch, lambda: step(lora), reps, 2, False)
             mode = f"eager ({type(exc).__name__} during capture)"
         out[name] = {"ms_per_step": round(ms, 3), "launch": mode}
     out["lora_overhead_ms"] = round(out["with_lora"]["ms_per_step"] - out["base_only"]["ms_per_step"], 3)
@@ -536,6 +543,10 @@ def bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, r
             out["config5_step"] = s5
         except Exception as exc:    # the headline does not depend on this leg
             out["config5_step"] = {"error": f"{type(exc).__name__}: {exc}"}
+        try:
+            out["decode_step"] = bench_config5_step(torch, W, dev, use_graph, decode_only=True)
+        except Exception as exc:
+            out["decode_step"] = {"error": f"{type(exc).__name__}: {exc}"}
     return out
 
 

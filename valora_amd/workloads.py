@@ -211,4 +211,14 @@ def config5_layer(hidden=4096, mlp=11008, len_div=1, n_decode=128, n_adapters=64
                    y0_random)
 
 
+def decode_layer(hidden=4096, mlp=11008, n_tokens=256, n_adapters=64, rank=16, y0_random=True, paged=True,
+                 targets=("q", "k", "v", "o", "gate", "up", "down")) -> Workload:
+    """The decode batch of configuration 2 (one token per request, Zipf(0.6) over 64 rank-16 adapters, fp16) with
+    LoRA on all seven projections of a decoder layer: what a decode-only serving step applies per layer."""
+    g = torch.Generator(device="cpu").manual_seed(1002)
+    req_ids = zipf_ids(n_adapters, n_tokens, 0.6, g)
+    pools = _layer_pools([rank] * n_adapters, hidden, mlp, torch.float16, g, targets, paged)
+    return _finish("decode_layer", torch.float16, req_ids, [1] * n_tokens, None, pools, g, y0_random)
+
+
 CONFIGS = {1: config1, 2: config2, 3: config3, 4: config4, 5: config5_layer}
