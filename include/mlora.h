@@ -57,11 +57,16 @@ enum {
   MLORA_ONE_LAUNCH_NO_WAIT = 4, /* with MLORA_ONE_LAUNCH: expand items do not wait at all and always
                                  compute their tile's partials themselves (the give-up path made
                                  testable; same results, slower)                                  */
-  MLORA_SHRINK_RECOMPUTE = 8  /* a split-K shrink of a small batch (tiles up to 64 tokens) sums its K
+  MLORA_SHRINK_RECOMPUTE = 8, /* a split-K shrink of a small batch (tiles up to 64 tokens) sums its K
                                  chunks inside the launch: the chunk of a tile that finishes last reads
                                  the others' partials out of the L2 it shares with them, or -- when they
                                  did not all run on its XCD -- computes them itself.  This flag makes
                                  every tile take the second path (made testable; same results, slower) */
+  MLORA_EXPAND_COLUMN_LOOP = 16 /* expand of a plan with 16-token expand tiles: a workgroup walks over two
+                                 256-column chunks of its tile instead of owning one.  The library does
+                                 this by itself where the grid would otherwise be several times what the
+                                 device holds (decode batches with many targets or wide outputs); the flag
+                                 forces it for any size (made testable; same results)                    */
 };
 
 /* What the kernels can vary per batch shape (see mlora_tile_lookup). */

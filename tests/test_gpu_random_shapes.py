@@ -181,3 +181,48 @@ def test_table_configurations_of_other_widths(dev, hidden, T, rank, n_adapters):
     want = O.lora_op(y0, x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, 0,
                      pool.a_scaling, n_slots=1)
     assert_parity(y.cpu(), want, what)
+
+
+@pytest.mark.parametrize("seed", range(300, 330))
+def test_expand_column_loop_gives_the_same_bits(dev, seed):
+    """The expand of 16-token tiles as one workgroup per (tile, 256-column chunk) and as one workgroup per two chunks
+    (what the library picks by itself for grids several times the device, forced here for any size): same bits, for
+    finished v and for split-K partials summed in the expand, one target and several, ranks up to 128, output widths
+    that end inside a chunk or leave the second chunk of a pair empty."""
+    rnd = random.Random(seed)
+    dtype = rnd.choice([torch.float16, torch.bfloat16])
+    T = rnd.choice([1, 3, 16, 17, 40, 100, 256, 300])
+    h_in = rnd.choice([256, 520, 1032, 4096])
+    h_out = rnd.choice([264, 512, 520, 768, 1000, 1032, 2056, 4096, 11008])
+    A = rnd.choice([1, 3, 9, 33, 70])
+    ranks = [rnd.choice([8, 16, 24, 32, 64, 128] if rnd.random() < 0.3 else [8, 16, 32]) for _ in range(A)]
+    ksplit = rnd.choice([1, 2, 4])
+    rie = ksplit > 1 and rnd.random() < 0.6
+    n_targets = rnd.choice([1, 1, 2, 3])
+    what = f"seed {seed}: {dtype} T={T} {h_in}->{h_out} A={A} ks={ksplit} rie={rie} targets={n_targets}"
+    print(what, flush=True)
+    g = torch.Generator().manual_seed(3000 + seed)
+    pool = W.make_pool(ranks, h_in, h_out, dtype, g, True, n_slots=4, std=0.05, heads=1)
+    ids = torch.randint(-1 if seed % 3 == 0 else 0, A, (T,), generator=g)
+    x = torch.randn(T, h_in, generator=g).to(dtype)
+    y0 = [torch.randn(T, h_out, generator=g).to(dtype) for _ in range(n_targets)]
+    pd = pool.to(dev)
+    idx = (pd.a_start, pd.a_len, pd.a_loc)
+    R = max(ranks)
+    kw = dict(hidden=h_in, bm_shrink=rnd.choice([16, 32]), bm_expand=16, ksplit=ksplit, reduce_in_expand=rie, one_launch=False)
+    outs = []
+    for loop in (False, True):
+        plan = LoraPlan(ids.to(dev), pd.a_start, pd.a_len, R, expand_column_loop=loop, **kw)
+        ys = [y.to(dev) for y in y0]
+        if n_targets == 1:
+            plan.apply(ys[0], x.to(dev), pd.key_buffer, pd.value_buffer, *idx, 2, pd.a_scaling)
+        else:
+            plan.apply_multi(ys, x.to(dev), pd.key_buffer, pd.value_buffer, *idx, list(range(n_targets)), pd.a_scaling)
+        outs.append([y.cpu() for y in ys])
+    for a, b in zip(*outs):
+        assert torch.equal(a, b), what
+    slot0 = 2 if n_targets == 1 else 0
+    want = O.lora_op(y0[0], x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, slot0,
+                     pool.a_scaling)
+    assert_parity(outs[1][0], want, what)
+    assert torch.equal(outs[1][0][ids < 0], y0[0][ids < 0])

@@ -348,6 +348,7 @@ int mlora_expand(void *stream, const mlora_plan *plan, void *y, int64_t T, int64
   a.kmax = (int)max_rank;
   a.slot = slot;
   a.n_ochunks = (int)((h_out + expand_bn() - 1) / expand_bn());
+  a.column_loop = (flags & MLORA_EXPAND_COLUMN_LOOP) ? 1 : 0;
   a.n_targets = 1;
   for (int i = 0; i < MLORA_MAX_TARGETS; ++i) {
     a.slots[i] = slot;
@@ -358,7 +359,7 @@ int mlora_expand(void *stream, const mlora_plan *plan, void *y, int64_t T, int64
   a.v_tstride = 0;
   a.partial_tstride = 0;
   return launch_expand((hipStream_t)stream, a, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand),
-                       dtype);
+                       plan->bm_expand, dtype);
 }
 
 int mlora_lora_apply(void *stream, const mlora_plan *plan, void *scratch, size_t scratch_nbytes, void *y,
@@ -492,6 +493,7 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
   e.kmax = (int)max_rank;
   e.slot = targets[0].slot;
   e.n_ochunks = (int)((h_out + expand_bn() - 1) / expand_bn());
+  e.column_loop = (flags & MLORA_EXPAND_COLUMN_LOOP) ? 1 : 0;
   e.n_targets = n_targets;
   for (int i = 0; i < MLORA_MAX_TARGETS; ++i) {
     const mlora_target &t = targets[i < n_targets ? i : 0];
@@ -520,7 +522,8 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
     d.resident = decode_resident;
     return launch_decode((hipStream_t)stream, d, (int)max_rank, dtype);
   }
-  return launch_expand((hipStream_t)stream, e, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand), dtype);
+  return launch_expand((hipStream_t)stream, e, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand),
+                       plan->bm_expand, dtype);
 }
 
 // ---- one-call entry points ------------------------------------------------------------------------

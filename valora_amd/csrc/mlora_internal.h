@@ -130,6 +130,7 @@ struct ExpandArgs {
   PoolDev pool;
   const uint16_t *scales;
   int T, h_out, kmax, slot, n_ochunks;
+  int column_loop;            // force the column-looping kernel for 16-token tiles (tests); else by grid size
 };
 
 
@@ -166,7 +167,7 @@ int launch_ids_from_requests(hipStream_t st, int64_t *ids_out, const int32_t *b_
 int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int64_t grid_tiles,
                   mlora_dtype dt);
 int launch_shrink_reduce(hipStream_t st, const ShrinkArgs &a, mlora_dtype dt);
-int launch_expand(hipStream_t st, const ExpandArgs &a, int max_rank, int64_t grid_tiles,
+int launch_expand(hipStream_t st, const ExpandArgs &a, int max_rank, int64_t grid_tiles, int bm_expand,
                   mlora_dtype dt);
 
 }  // namespace mlora
