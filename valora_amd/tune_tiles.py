@@ -48,10 +48,11 @@ def _time(fn, reps=30, warm=3) -> float:
 
 
 def synthetic_batch(n_tokens: int, n_adapters: int, rank: int, hidden: int, dtype, seed: int):
-    """Decode-like (one token per request) up to 1024 tokens, 128-token requests above; adapters drawn
-    Zipf(0.7) per request."""
+    """Decode-like (one token per request) up to 1024 tokens; above, requests of 128 tokens, or shorter ones where
+    that many would be fewer than the adapter bucket stands for (2048 tokens over 128 adapters: 16-token requests,
+    the decode-heavy mix of a continuous batch); adapters drawn Zipf(0.7) per request."""
     g = torch.Generator().manual_seed(seed)
-    req_len = 1 if n_tokens <= 1024 else 128
+    req_len = 1 if n_tokens <= 1024 else min(128, max(1, n_tokens // max(1, n_adapters)))
     n_req = max(1, n_tokens // req_len)
     req_ids = W.zipf_ids(n_adapters, n_req, 0.7, g)
     ids = torch.repeat_interleave(req_ids, req_len)
@@ -133,7 +134,7 @@ def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--overwrite", action="store_true")
     ap.add_argument("--hidden", type=int, nargs="+", default=[4096])
-    ap.add_argument("--tokens", type=int, nargs="+", default=[8, 64, 256, 1024, 4096, 16384])
+    ap.add_argument("--tokens", type=int, nargs="+", default=[8, 64, 128, 256, 512, 1024, 2048, 4096, 16384])
     ap.add_argument("--adapters", type=int, nargs="+", default=[8, 32, 128])
     ap.add_argument("--ranks", type=int, nargs="+", default=list(tt.RANK_BUCKETS))
     ap.add_argument("--out", default=tt.TABLE_PATH)
