@@ -93,7 +93,14 @@ mlora_tile_config tile_lookup(int64_t T, int64_t max_rank, int64_t hidden, int64
       return memo[i].cfg;
   mlora_tile_config c;
   // the rule for shapes without an entry looks at T and A themselves, not at their buckets: not remembered
-  if (!table_lookup(max_rank, hidden, tb, rb, ab, c)) return tile_fallback(T, max_rank, hidden, A);
+  // an adapter bucket without entries takes those of the next larger measured one, else of the next smaller
+  bool found = table_lookup(max_rank, hidden, tb, rb, ab, c);
+  constexpr int NA = (int)(sizeof(kAdapterBuckets) / sizeof(kAdapterBuckets[0]));
+  for (int i = 0; i < NA && !found; ++i)
+    if (kAdapterBuckets[i] > ab) found = table_lookup(max_rank, hidden, tb, rb, kAdapterBuckets[i], c);
+  for (int i = NA - 1; i >= 0 && !found; --i)
+    if (kAdapterBuckets[i] < ab) found = table_lookup(max_rank, hidden, tb, rb, kAdapterBuckets[i], c);
+  if (!found) return tile_fallback(T, max_rank, hidden, A);
   memo[next] = Memo{tb, rb, hidden, ab, c, true};
   next = (next + 1) % N_MEMO;
   return c;

@@ -48,6 +48,7 @@ class LoraPlan:
         rie = cfg.reduce_in_expand if reduce_in_expand is None else reduce_in_expand
         self.flags = _lib.REDUCE_IN_EXPAND if rie else 0
         self.one_launch = bool(cfg.one_launch if one_launch is None else one_launch)
+        self._one_launch_by_table = one_launch is None
         if self.one_launch and (self.max_rank > 64 or bm_shrink not in (None, 16) or bm_expand not in (None, 16)):
             if one_launch:
                 raise RuntimeError("No suitable kernel. the one-launch op needs 16-token tiles and max_rank <= 64")
@@ -177,9 +178,18 @@ class LoraPlan:
         tg = (_lib.Target * n)()
         for i in range(n):
             tg[i] = _lib.Target(_lib.ptr(ys[i]), _lib.ptr(vbs[i]), vbs[i].numel() // h_out, int(slots[i]))
+        flags = self.flags
+        if self.one_launch and self._one_launch_by_table and n > 1:
+            # the table's mark was measured on one target.  With several, the one-launch op still pays up to 16
+            # expand items per tile (two 4096-wide targets: 6.5-7.9 us against 7.5-9.2 as two launches, 1-64 tokens);
+            # beyond that two launches win (three rank-64 targets of 8 tokens: 15.0 against 18.3 us, gate+up 4096 ->
+            # 11008: 7.9 against 8.9).  Same tiles, same split, same bits either way.
+            chunk = 512 if self.max_rank <= 32 else 256
+            if n * ((h_out + chunk - 1) // chunk) > 16:
+                flags &= ~(_lib.ONE_LAUNCH | _lib.ONE_LAUNCH_NO_WAIT)
         _lib.check(_lib.lib().mlora_lora_apply_multi(
             _lib.current_stream(self.device), self.handle, _lib.ptr(self.scratch), self.scratch.numel(), _lib.ptr(x),
-            self.T, h_in, h_out, self.max_rank, pa, n, tg, _lib.ptr(scales), int(self.ksplit), self.flags,
+            self.T, h_in, h_out, self.max_rank, pa, n, tg, _lib.ptr(scales), int(self.ksplit), flags,
             _lib.dtype_code(x.dtype)))
 
     def apply(self, y: torch.Tensor, x: torch.Tensor, key_buffer: torch.Tensor, value_buffer: torch.Tensor,
