@@ -153,6 +153,11 @@ TABLE_CASES = [
     (2048, 8, 16, 8), (2048, 256, 32, 32), (2048, 3000, 64, 8), (3072, 60, 64, 8), (3072, 1024, 16, 100),
     (7168, 7, 32, 8), (7168, 256, 16, 32), (7168, 2500, 128, 8), (14336, 64, 16, 32), (14336, 1500, 64, 8),
     (28672, 8, 16, 8), (28672, 200, 32, 8), (28672, 1100, 64, 8),
+    # one adapter for the whole batch, and the 128- / 512- / 2048-token buckets
+    (4096, 1, 16, 1), (4096, 100, 64, 1), (4096, 500, 16, 1), (4096, 1500, 32, 1), (4096, 5000, 64, 1), (4096, 700, 128, 1),
+    (11008, 300, 16, 1), (11008, 2000, 64, 1), (8192, 120, 32, 1), (2048, 1300, 16, 1), (28672, 400, 16, 1),
+    (4096, 100, 16, 100), (4096, 400, 32, 32), (4096, 1500, 16, 100), (4096, 2000, 64, 32), (11008, 500, 64, 8),
+    (4096, 300, 16, 500),
 ]
 
 
@@ -163,7 +168,7 @@ def test_table_configurations_of_other_widths(dev, hidden, T, rank, n_adapters):
     from valora_amd import tile_table
     g = torch.Generator().manual_seed(hidden + T + rank)
     dtype = torch.bfloat16 if (T + rank) % 32 else torch.float16
-    h_out = 4096 if hidden > 8192 else hidden          # 13824 and wider are MLP widths: down-projection shape
+    h_out = 4096 if hidden > 8192 else hidden          # 11008 and wider are MLP widths: down-projection shape
     pool = W.make_pool([rank] * n_adapters, hidden, h_out, dtype, g, True, n_slots=1, std=0.03, heads=1)
     req = 1 if T <= 1024 else 128
     ids = torch.repeat_interleave(W.zipf_ids(n_adapters, (T + req - 1) // req, 0.7, g), req)[:T]
