@@ -436,6 +436,36 @@ def bench_adapter_residency(torch, dev):
     return out
 
 
+def bench_byte_heavy_decode(torch, W, LoraPlan, dev, use_graph, reps):
+    """Decode batches (one token per request, 4096 -> 4096, fp16, adapters drawn Zipf(0.7) over 128) whose adapters
+    weigh a few hundred MB: the same kernels as the headline, where the op is long enough for its bytes to decide.
+    Bytes are algorithmic: x + y read + y write + A and B of the adapters the batch really touches."""
+    out = []
+    H = 4096
+    for T, A, r in ((256, 128, 64), (512, 128, 128), (1024, 128, 64), (1024, 128, 128)):
+        g = torch.Generator().manual_seed(T + A + r)
+        ids = W.zipf_ids(A, T, 0.7, g)
+        pool = W.make_pool([r] * A, H, H, torch.float16, g, True, n_slots=1).to(dev)
+        x = torch.randn(T, H, generator=g).half().to(dev)
+        ys = [torch.zeros(T, H, dtype=torch.float16, device=dev) for _ in range(4)]
+        plan = LoraPlan(ids.to(dev), pool.a_start, pool.a_len, r, n_slots=1, hidden=H)
+
+        def run():
+            for y in ys:
+                plan.apply(y, x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, 0, pool.a_scaling)
+
+        ms, _ = time_graph(torch, run, max(10, reps // 4), 3, use_graph)
+        us = ms * 1e3 / len(ys)
+        touched = len(set(ids.tolist()))
+        nbytes = 3 * T * H * 2 + 2 * touched * r * H * 2
+        out.append({"tokens": T, "rank": r, "adapters_touched": touched, "us": round(us, 2), "bytes": nbytes,
+                    "gbps": round(nbytes / us / 1e3, 1), "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 3),
+                    "tile": [plan.bm_shrink, plan.ksplit, plan.bm_expand], "one_launch": plan.one_launch})
+        del pool, x, ys, plan
+        torch.cuda.empty_cache()
+    return out
+
+
 def bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, reps, no_step5):
     """Legs beside the headline, all on the config-2 decode shape with the same rotation over `L` layers'
     buffers: a whole attention block's LoRA work per layer, and the same shrink + expand pair reached through
@@ -537,6 +567,10 @@ def bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, r
     out["dropin_pair_is"] = ("shrink + expand of the config-2 op through the reference's own entry points (two calls per "
                              "layer, torch binding -> one C-ABI call each with the cached plan of the batch); graph = HIP "
                              "graph replay, eager = launched from Python call by call (events / host wall clock)")
+    try:
+        out["byte_heavy_decode"] = bench_byte_heavy_decode(torch, W, LoraPlan, dev, use_graph, reps)
+    except Exception as exc:    # the headline does not depend on this leg
+        out["byte_heavy_decode"] = {"error": f"{type(exc).__name__}: {exc}"}
     if not no_step5:
         try:
             s5 = bench_config5_step(torch, W, dev, use_graph)
