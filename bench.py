@@ -466,6 +466,46 @@ def bench_byte_heavy_decode(torch, W, LoraPlan, dev, use_graph, reps):
     return out
 
 
+def bench_single_adapter_vs_gemm(torch, W, LoraPlan, dev, use_graph, reps):
+    """One adapter for the whole batch: the op is then two dense skinny matrix products, y += s * (x @ A^T) @ B, which
+    the vendor's GEMM library can do as torch.mm + Tensor.addmm_ (operands laid out the way the library likes them).
+    A yardstick from outside this code base for what the device gives on these shapes; 4096 -> 4096, fp16."""
+    out = []
+    H, n = 4096, 8
+    for T, r in ((256, 16), (256, 64), (4096, 16), (4096, 64), (16384, 16), (16384, 64)):
+        g = torch.Generator().manual_seed(T + r)
+        pool = W.make_pool([r], H, H, torch.float16, g, False, n_slots=1, heads=1).to(dev)
+        ids = torch.zeros(T, dtype=torch.long, device=dev)
+        gd = torch.Generator(device=dev).manual_seed(T + r)
+        xs = [torch.randn(T, H, generator=gd, device=dev).half() for _ in range(n)]
+        ys = [torch.randn(T, H, generator=gd, device=dev).half() for _ in range(n)]
+        vs = [torch.empty(T, r, dtype=torch.float16, device=dev) for _ in range(n)]
+        a_t = (torch.randn(H, r, generator=gd, device=dev) * 0.02).half()
+        b = (torch.randn(r, H, generator=gd, device=dev) * 0.02).half()
+        plan = LoraPlan(ids, pool.a_start, pool.a_len, r, n_slots=1, hidden=H)
+
+        def ours():
+            for l in range(n):
+                plan.apply(ys[l], xs[l], pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, 0,
+                           pool.a_scaling)
+
+        def gemm():
+            for l in range(n):
+                torch.mm(xs[l], a_t, out=vs[l])
+                ys[l].addmm_(vs[l], b, alpha=0.5)
+
+        k = max(10, reps // 4)
+        us_ours = time_graph(torch, ours, k, 3, use_graph)[0] * 1e3 / n
+        us_gemm = time_graph(torch, gemm, k, 3, use_graph)[0] * 1e3 / n
+        nbytes = (3 * T * H + 2 * r * H) * 2
+        out.append({"tokens": T, "rank": r, "us": round(us_ours, 2), "torch_mm_addmm_us": round(us_gemm, 2),
+                    "gbps": round(nbytes / us_ours / 1e3, 1), "tile": [plan.bm_shrink, plan.ksplit, plan.bm_expand],
+                    "one_launch": plan.one_launch})
+        del pool, xs, ys, vs, plan
+        torch.cuda.empty_cache()
+    return out
+
+
 def bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, reps, no_step5):
     """Legs beside the headline, all on the config-2 decode shape with the same rotation over `L` layers'
     buffers: a whole attention block's LoRA work per layer, and the same shrink + expand pair reached through
@@ -571,6 +611,10 @@ def bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, r
         out["byte_heavy_decode"] = bench_byte_heavy_decode(torch, W, LoraPlan, dev, use_graph, reps)
     except Exception as exc:    # the headline does not depend on this leg
         out["byte_heavy_decode"] = {"error": f"{type(exc).__name__}: {exc}"}
+    try:
+        out["single_adapter_vs_gemm"] = bench_single_adapter_vs_gemm(torch, W, LoraPlan, dev, use_graph, reps)
+    except Exception as exc:
+        out["single_adapter_vs_gemm"] = {"error": f"{type(exc).__name__}: {exc}"}
     if not no_step5:
         try:
             s5 = bench_config5_step(torch, W, dev, use_graph)

@@ -93,11 +93,41 @@ def tune_shape(dev, n_tokens, n_adapters, rank, hidden, dtype=torch.float16, cop
             best = (us, bm, ks, rie)
     _, bm, ks, rie = best
     best_e = None
-    for be in (16, 32, 64, 128, 256):
+    for be in EXPAND_HEIGHTS if n_tokens > 1024 else (16, 32, 64, 128, 256):
         us = op_us(bm, ks, be, rie)
         if better(us, best_e):
             best_e = (us, be)
     return {"bm_shrink": bm, "ksplit": ks, "bm_expand": best_e[1], "reduce_in_expand": bool(rie)}, best_e[0]
+
+
+EXPAND_HEIGHTS = (16, 32, 48, 64, 96, 128, 192, 256)
+
+
+def tune_expand_height(dev, n_tokens, n_adapters, rank, hidden, entry, dtype=torch.float16, copies=4):
+    """The expand tile height of an existing entry swept again over EXPAND_HEIGHTS (shrink tiles, split-K and who
+    sums the chunks stay): returns the entry to keep, its time and the old entry's time."""
+    ids, pool, x = synthetic_batch(n_tokens, n_adapters, rank, hidden, dtype, seed=n_tokens + n_adapters + rank)
+    ids, x, p = ids.to(dev), x.to(dev), pool.to(dev)
+    ys = [torch.zeros(ids.numel(), hidden, dtype=dtype, device=dev) for _ in range(copies)]
+    idx = (p.a_start, p.a_len, p.a_loc)
+
+    def op_us(be):
+        plan = LoraPlan(ids, p.a_start, p.a_len, rank, hidden=hidden, bm_shrink=entry["bm_shrink"], ksplit=entry["ksplit"],
+                        bm_expand=be, reduce_in_expand=entry.get("reduce_in_expand", False), one_launch=False)
+        return _time(lambda: [plan.apply(y, x, p.key_buffer, p.value_buffer, *idx, 0, p.a_scaling)
+                              for y in ys]) / copies
+
+    old = op_us(entry["bm_expand"])
+    best = (old, entry["bm_expand"])
+    for be in EXPAND_HEIGHTS:
+        if be == entry["bm_expand"]:
+            continue
+        us = op_us(be)
+        if us < 0.97 * best[0]:
+            best = (us, be)
+    new = dict(entry)
+    new["bm_expand"] = best[1]
+    return new, best[0], old
 
 
 def tune_one_launch(dev, n_tokens, n_adapters, rank, hidden, entry, dtype=torch.float16, copies=4):
@@ -141,6 +171,9 @@ def main():
     ap.add_argument("--one-launch", action="store_true",
                     help="revisit the existing entries of decode-like shapes (<= 1024 tokens, rank <= 64; the protected "
                          "ones too) and mark those where the one-launch op is faster than the entry's two launches")
+    ap.add_argument("--expand-heights", action="store_true",
+                    help="revisit the expand tile height of the existing entries above 1024 tokens over the finer list "
+                         "(48, 96 and 192 tokens as well); protected and one-launch entries stay")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("tune_tiles needs a GPU")
@@ -151,6 +184,16 @@ def main():
     t0 = time.time()
     for hidden, n_tokens, n_adapters, rank in itertools.product(args.hidden, args.tokens, args.adapters, args.ranks):
         k = tt.key(n_tokens, rank, hidden, n_adapters)
+        if args.expand_heights:
+            e = entries.get(k)
+            if e and n_tokens > 1024 and not e.get("one_launch") and k not in table.get("protected", []):
+                entries[k], us, old = tune_expand_height(dev, n_tokens, min(n_adapters, max(1, n_tokens)), rank, hidden, e)
+                print(f"{k:24s} expand tile {e['bm_expand']} ({old:.1f} us) -> {entries[k]['bm_expand']} ({us:.1f} us)  "
+                      f"[{time.time() - t0:.0f} s]", flush=True)
+                torch.cuda.empty_cache()
+                with open(args.out, "w") as f:
+                    json.dump(table, f, indent=1)
+            continue
         if args.one_launch:
             if k in entries and n_tokens <= 1024 and rank <= 64:
                 new, two, one = tune_one_launch(dev, n_tokens, min(n_adapters, max(1, n_tokens)), rank, hidden, entries[k])
