@@ -71,7 +71,7 @@ enum {
 
 /* What the kernels can vary per batch shape (see mlora_tile_lookup). */
 typedef struct {
-  int32_t bm_shrink;        /* tokens per shrink tile: 16, 32, 64 (direct loads) or 128 (LDS-staged)  */
+  int32_t bm_shrink;        /* tokens per shrink tile: 16, 32, 64 (direct loads), 128 or 256 (LDS-staged) */
   int32_t ksplit;           /* K chunks the shrink is split into                                      */
   int32_t bm_expand;        /* tokens per expand tile: multiple of 16 up to 256                       */
   int32_t flags;            /* MLORA_REDUCE_IN_EXPAND | MLORA_ONE_LAUNCH                              */
@@ -139,7 +139,7 @@ int mlora_tile_fallback(int64_t n_tokens, int64_t max_rank, int64_t hidden, int6
  * [0, n_adapters) or an adapter of rank 0 marks a token that gets no LoRA).  Stable counting
  * sort of the tokens by adapter + one tile list per tile height.  Replaces the host-side
  * grouping done by precompute_sgmm_args_* (atmm/valora/csrc/bgmv/bgmv_impl.cuh:76-125).
- * bm_shrink, bm_expand: tile heights in tokens (16, 32, 64 or 128 / any multiple of 16 up to 256);
+ * bm_shrink, bm_expand: tile heights in tokens (16, 32, 64, 128 or 256 -- 256 up to rank 64 -- / any multiple of 16 up to 256);
  * 0 lets the library choose.                                                                 */
 int mlora_build_plan(void *stream, mlora_plan *plan, const int64_t *ids, int64_t T,
                      const int64_t *a_start, const int64_t *a_len, int64_t n_adapters,

@@ -111,7 +111,7 @@ def test_tile_lookup_through_the_c_abi_agrees_with_the_json_table():
 def test_tile_table_lookup_and_fallback():
     from valora_amd import tile_table as tt
     cfg = tt.lookup(256, 16, 4096, 64)
-    assert cfg.bm_shrink in (16, 32, 64, 128) and 1 <= cfg.ksplit <= 64 and cfg.bm_expand % 16 == 0
+    assert cfg.bm_shrink in (16, 32, 64, 128, 256) and 1 <= cfg.ksplit <= 64 and cfg.bm_expand % 16 == 0
     fb = tt.fallback(100000, 128, 4096, 4)          # long runs per adapter -> LDS-staged 128-token tiles
     assert fb.bm_shrink == 128 and fb.ksplit >= 1 and not fb.reduce_in_expand
     fb = tt.fallback(300, 64, 4096, 200)            # decode-like -> direct 16-token tiles, expand sums the chunks
@@ -121,7 +121,7 @@ def test_tile_table_lookup_and_fallback():
     for rank in (8, 40, 128):                       # every table entry is a configuration the kernels take
         for T in (1, 300, 5000, 100000):
             c = tt.lookup(T, rank, 4096, 16)
-            assert c.bm_shrink in (16, 32, 64, 128) and not (rank > 64 and c.bm_shrink == 64)
+            assert c.bm_shrink in (16, 32, 64, 128, 256) and not (rank > 64 and c.bm_shrink in (64, 256))
             assert 1 <= c.ksplit <= 64 and c.bm_expand % 16 == 0 and 16 <= c.bm_expand <= 256
 
 

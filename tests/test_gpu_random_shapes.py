@@ -28,10 +28,10 @@ def draw(seed):
     big = rnd.random() < 0.25
     ranks = [rnd.choice(RANKS if big else RANKS[:6]) for _ in range(n_adapters)]
     n_slots = rnd.choice([1, 2, 4, 4, 5])
-    cfg = dict(bm_shrink=rnd.choice([16, 32, 64, 128]), bm_expand=rnd.choice([16, 32, 48, 64, 96, 128, 192, 256]),
+    cfg = dict(bm_shrink=rnd.choice([16, 32, 64, 128, 256]), bm_expand=rnd.choice([16, 32, 48, 64, 96, 128, 192, 256]),
                ksplit=rnd.choice([1, 2, 3, 4, 8]), reduce_in_expand=rnd.random() < 0.5)
-    if max(ranks) > 64 and cfg["bm_shrink"] == 64:
-        cfg["bm_shrink"] = 32       # ranks above 64 have no 64-token shrink tile (the library says so)
+    if max(ranks) > 64 and cfg["bm_shrink"] in (64, 256):
+        cfg["bm_shrink"] //= 2      # ranks above 64 have no 64- or 256-token shrink tile (the library says so)
     style = rnd.choice(["random", "sorted", "holes", "one", "none"])
     return dtype, T, h_in, h_out, ranks, n_slots, cfg, style
 

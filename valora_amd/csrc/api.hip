@@ -196,8 +196,8 @@ int mlora_build_plan(void *stream, mlora_plan *plan, const int64_t *ids, int64_t
     if (bm_shrink == 0) bm_shrink = c.bm_shrink;
     if (bm_expand == 0) bm_expand = c.bm_expand;
   }
-  if (bm_shrink != 16 && bm_shrink != 32 && bm_shrink != 64 && bm_shrink != 128)
-    return fail(MLORA_ERR_NO_KERNEL, "build_plan: bm_shrink=%d not in {16,32,64,128}", bm_shrink);
+  if (bm_shrink != 16 && bm_shrink != 32 && bm_shrink != 64 && bm_shrink != 128 && bm_shrink != 256)
+    return fail(MLORA_ERR_NO_KERNEL, "build_plan: bm_shrink=%d not in {16,32,64,128,256}", bm_shrink);
   if (bm_expand < 16 || bm_expand > 256 || (bm_expand % 16) != 0)
     return fail(MLORA_ERR_NO_KERNEL, "build_plan: bm_expand=%d not a multiple of 16 in [16,256]", bm_expand);
   const PlanLayout L = plan_layout(T, n_adapters);

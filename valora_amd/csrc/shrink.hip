@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256) void shrink_kernel(const int32_t *tiles_base, 
 // lane that fills 16-byte chunk c of row R fetches global chunk c ^ (R & 7), which spreads the
 // later ds_read_b128 of an MFMA operand (16 rows, one chunk column) over the banks.  Two stages
 // are always in flight while the third is consumed; one s_barrier per K step.
-template <typename T, int NB>
+template <typename T, int NB, int MBW>
 __global__ __launch_bounds__(256) void shrink_gemm_kernel(const int32_t *tiles_base, int h_ksplit, int h_n_targets, int, int,
                                                           ShrinkArgs args_in) {
   // workgroup id = (tile * targets + target) * ksplit + K chunk.  The id mod 8 selects the XCD, so
@@ -252,14 +252,14 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(const int32_t *tiles_b
   const int s = blockIdx.x - wg_tz * h_ksplit;
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
-  constexpr int MBW = 2, KC = 64, KS = KC / 32, STAGES = 3;
+  constexpr int KC = 64, KS = KC / 32, STAGES = 3;      // MBW: 16-token blocks per wave (tile = 64 * MBW tokens)
   static_assert(KC * 2 == 128, "a K step is one 128-byte line per row");
   constexpr int XBLK = MBW * 2;                         // 8-row groups (1 KB) of x per wave per stage
   constexpr int ABLK = NB * 2;                          // 8-row groups of A per stage (shared)
   constexpr int APW = ABLK >= 4 ? ABLK / 4 : 1;         // A groups each wave loads per stage
   constexpr int A_SLOTS = APW * 4;                      // >= ABLK; surplus slots hold duplicates
   constexpr int STAGE_BYTES = (4 * XBLK + A_SLOTS) * 1024;
-  constexpr int TILE_BYTES = 128 * NB * 16 * 4;
+  constexpr int TILE_BYTES = 64 * MBW * NB * 16 * 4;
   constexpr int LOADS_PER_STAGE = XBLK + APW;           // per wave, identical for all waves
   constexpr int RING_BYTES = STAGES * STAGE_BYTES + 1024;   // + one scratch block for dummy loads
   __shared__ __align__(16) unsigned char s_raw[RING_BYTES > TILE_BYTES ? RING_BYTES : TILE_BYTES];
@@ -408,13 +408,18 @@ __global__ __launch_bounds__(256) void shrink_gemm_kernel(const int32_t *tiles_b
   shrink_epilogue<T>(p, otile, NB * 16, s, pos0, cnt, r, perm);
 }
 
-template <typename T>
+template <typename T, int MBW>
 int launch_gemm_nb(hipStream_t st, const ShrinkArgs &a, int nb, dim3 grid) {
   switch (nb) {
-    case 1: hipLaunchKernelGGL((shrink_gemm_kernel<T, 1>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
-    case 2: hipLaunchKernelGGL((shrink_gemm_kernel<T, 2>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
-    case 4: hipLaunchKernelGGL((shrink_gemm_kernel<T, 4>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
-    case 8: hipLaunchKernelGGL((shrink_gemm_kernel<T, 8>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
+    case 1: hipLaunchKernelGGL((shrink_gemm_kernel<T, 1, MBW>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
+    case 2: hipLaunchKernelGGL((shrink_gemm_kernel<T, 2, MBW>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
+    case 4: hipLaunchKernelGGL((shrink_gemm_kernel<T, 4, MBW>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a); break;
+    case 8:
+      if constexpr (MBW <= 2) {
+        hipLaunchKernelGGL((shrink_gemm_kernel<T, 8, MBW>), grid, dim3(256), 0, st, a.plan + a.off_tiles, a.ksplit, a.n_targets, a.reduce_here, a.n_tiles, a);
+        break;
+      }
+      return fail(MLORA_ERR_NO_KERNEL, "shrink: rank > 64 has no 256-token tile");
     default: return fail(MLORA_ERR_NO_KERNEL, "shrink: no kernel for rank blocks=%d", nb);
   }
   return check_launch("shrink_gemm_kernel");
@@ -438,8 +443,9 @@ int launch_shrink_t(hipStream_t st, const ShrinkArgs &a, int bm, int nb, dim3 gr
     case 16: return launch_shrink_nb<T, 1>(st, a, nb, grid);
     case 32: return launch_shrink_nb<T, 2>(st, a, nb, grid);
     case 64: return launch_shrink_nb<T, 4>(st, a, nb, grid);
-    case 128: return launch_gemm_nb<T>(st, a, nb, grid);
-    default: return fail(MLORA_ERR_NO_KERNEL, "shrink: tile height %d not in {16,32,64,128}", bm);
+    case 128: return launch_gemm_nb<T, 2>(st, a, nb, grid);
+    case 256: return launch_gemm_nb<T, 4>(st, a, nb, grid);
+    default: return fail(MLORA_ERR_NO_KERNEL, "shrink: tile height %d not in {16,32,64,128,256}", bm);
   }
 }
 
@@ -461,7 +467,7 @@ int launch_shrink(hipStream_t st, const ShrinkArgs &a, int bm, int max_rank, int
                   mlora_dtype dt) {
   int nb = (max_rank + 15) / 16;
   nb = nb <= 1 ? 1 : nb <= 2 ? 2 : nb <= 4 ? 4 : 8;
-  if (nb == 8 && bm == 64) return fail(MLORA_ERR_NO_KERNEL, "shrink: rank > 64 needs tile height 16, 32 or 128");
+  if (nb == 8 && (bm == 64 || bm == 256)) return fail(MLORA_ERR_NO_KERNEL, "shrink: rank > 64 needs tile height 16, 32 or 128");
   if (grid_tiles <= 0) return MLORA_OK;
   if (a.reduce_here) grid_tiles = (grid_tiles + 7) / 8 * 8;   // ids are dealt to the 8 XCDs tile by tile
   if (grid_tiles * a.ksplit * a.n_targets > 0x7fffffff) return fail(MLORA_ERR_NO_KERNEL, "shrink: grid too large");

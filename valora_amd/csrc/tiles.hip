@@ -134,6 +134,7 @@ static bool table_lookup(int64_t max_rank, int64_t hidden, int64_t tb, int64_t r
   }
   if (max_rank > 64) {
     if (c.bm_shrink == 64) c.bm_shrink = 32;   // ranks above 64 have no 64-token shrink tile
+    if (c.bm_shrink == 256) c.bm_shrink = 128;  // and no 256-token one
     c.flags &= ~MLORA_ONE_LAUNCH;
   }
   if (c.flags & MLORA_ONE_LAUNCH) c.flags |= MLORA_REDUCE_IN_EXPAND;

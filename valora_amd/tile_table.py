@@ -26,7 +26,7 @@ RANK_BUCKETS = (16, 32, 64, 128)
 
 @dataclass(frozen=True)
 class TileConfig:
-    bm_shrink: int   # tokens per shrink tile: 16, 32, 64 (direct loads) or 128 (weights staged in LDS)
+    bm_shrink: int   # tokens per shrink tile: 16, 32, 64 (direct loads), 128 or 256 (weights staged in LDS)
     ksplit: int      # K-chunks the shrink is split into (partials summed by the consumer)
     bm_expand: int   # tokens per expand tile: multiple of 16 up to 256
     reduce_in_expand: bool = False  # split-K chunks summed by the expand launch (small batches)

@@ -79,12 +79,12 @@ def tune_shape(dev, n_tokens, n_adapters, rank, hidden, dtype=torch.float16, cop
         return _time(lambda: [plan.apply(y, x, p.key_buffer, p.value_buffer, *idx, 0, p.a_scaling)
                               for y in ys]) / copies
 
-    heights = (16, 32) if n_tokens <= 256 else (16, 32, 64, 128)
+    heights = (16, 32) if n_tokens <= 256 else (16, 32, 64, 128) if n_tokens <= 4096 else (16, 32, 64, 128, 256)
     splits = (4, 8, 16, 32, 2, 1) if n_tokens <= 1024 else (4, 8, 16, 2, 1)
     be0 = 16 if n_tokens <= 1024 else 64
     best = None
     for bm, ks, rie in itertools.product(heights, splits, (False, True)):
-        if (rank > 64 and bm == 64) or (rie and ks == 1) or ks * 128 > hidden:
+        if (rank > 64 and bm in (64, 256)) or (rie and ks == 1) or ks * 128 > hidden:
             continue
         if rie and n_tokens > 4096:        # the partials are re-read once per column chunk: never pays there
             continue
@@ -130,6 +130,33 @@ def tune_expand_height(dev, n_tokens, n_adapters, rank, hidden, entry, dtype=tor
     return new, best[0], old
 
 
+def tune_tall_shrink(dev, n_tokens, n_adapters, rank, hidden, entry, dtype=torch.float16, copies=4):
+    """Does a 256-token shrink tile (half the re-reads of A, one workgroup per compute unit) beat an entry that uses
+    128-token tiles?  Split-K 4 and 8 are tried with the entry's expand tile; returns the entry to keep and both times."""
+    ids, pool, x = synthetic_batch(n_tokens, n_adapters, rank, hidden, dtype, seed=n_tokens + n_adapters + rank)
+    ids, x, p = ids.to(dev), x.to(dev), pool.to(dev)
+    ys = [torch.zeros(ids.numel(), hidden, dtype=dtype, device=dev) for _ in range(copies)]
+    idx = (p.a_start, p.a_len, p.a_loc)
+
+    def op_us(bm, ks):
+        plan = LoraPlan(ids, p.a_start, p.a_len, rank, hidden=hidden, bm_shrink=bm, ksplit=ks, bm_expand=entry["bm_expand"],
+                        reduce_in_expand=False, one_launch=False)
+        return _time(lambda: [plan.apply(y, x, p.key_buffer, p.value_buffer, *idx, 0, p.a_scaling)
+                              for y in ys]) / copies
+
+    old = op_us(entry["bm_shrink"], entry["ksplit"])
+    best = (old, entry["bm_shrink"], entry["ksplit"])
+    for ks in (4, 8, 2):
+        if ks * 128 > hidden:
+            continue
+        us = op_us(256, ks)
+        if us < 0.97 * best[0]:
+            best = (us, 256, ks)
+    new = dict(entry)
+    new["bm_shrink"], new["ksplit"] = best[1], best[2]
+    return new, best[0], old
+
+
 def tune_one_launch(dev, n_tokens, n_adapters, rank, hidden, entry, dtype=torch.float16, copies=4):
     """Does the one-launch op (shrink and expand items of one grid, 16-token tiles) beat the two-launch entry of
     this shape?  Returns the entry to keep and both timings.  Only decode-like shapes qualify: rank <= 64 and a
@@ -171,6 +198,9 @@ def main():
     ap.add_argument("--one-launch", action="store_true",
                     help="revisit the existing entries of decode-like shapes (<= 1024 tokens, rank <= 64; the protected "
                          "ones too) and mark those where the one-launch op is faster than the entry's two launches")
+    ap.add_argument("--tall-shrink", action="store_true",
+                    help="revisit the existing entries above 4096 tokens that use 128-token shrink tiles (rank <= 64, summed "
+                         "by the reduce launch): 256-token tiles where they are faster; protected entries stay")
     ap.add_argument("--expand-heights", action="store_true",
                     help="revisit the expand tile height of the existing entries above 1024 tokens over the finer list "
                          "(48, 96 and 192 tokens as well); protected and one-launch entries stay")
@@ -184,6 +214,17 @@ def main():
     t0 = time.time()
     for hidden, n_tokens, n_adapters, rank in itertools.product(args.hidden, args.tokens, args.adapters, args.ranks):
         k = tt.key(n_tokens, rank, hidden, n_adapters)
+        if args.tall_shrink:
+            e = entries.get(k)
+            if (e and n_tokens > 4096 and rank <= 64 and e["bm_shrink"] == 128 and not e.get("reduce_in_expand")
+                    and k not in table.get("protected", [])):
+                entries[k], us, old = tune_tall_shrink(dev, n_tokens, min(n_adapters, max(1, n_tokens)), rank, hidden, e)
+                print(f"{k:24s} shrink tile 128 x {e['ksplit']} ({old:.1f} us) -> {entries[k]['bm_shrink']} x "
+                      f"{entries[k]['ksplit']} ({us:.1f} us)  [{time.time() - t0:.0f} s]", flush=True)
+                torch.cuda.empty_cache()
+                with open(args.out, "w") as f:
+                    json.dump(table, f, indent=1)
+            continue
         if args.expand_heights:
             e = entries.get(k)
             if e and n_tokens > 1024 and not e.get("one_launch") and k not in table.get("protected", []):
