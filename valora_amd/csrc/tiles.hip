@@ -24,7 +24,7 @@ const Entry kTable[] = {
 };
 constexpr int kEntries = (int)(sizeof(kTable) / sizeof(kTable[0]));
 
-const int64_t kTokenBuckets[] = {8, 64, 128, 256, 512, 1024, 2048, 4096, 16384, (int64_t)1 << 22};
+const int64_t kTokenBuckets[] = {8, 64, 128, 256, 512, 1024, 2048, 4096, 8192, 16384, (int64_t)1 << 22};
 const int64_t kAdapterBuckets[] = {1, 8, 32, 128, 8192};
 const int64_t kRankBuckets[] = {16, 32, 64, 128};
 
@@ -88,9 +88,15 @@ mlora_tile_config tile_lookup(int64_t T, int64_t max_rank, int64_t hidden, int64
   constexpr int N_MEMO = 8;
   static thread_local Memo memo[N_MEMO];
   static thread_local int next = 0;
+  // what depends on T itself rather than on its bucket: a 256-token shrink tile needs a batch that fills the device
+  // with such tiles (one workgroup per compute unit); the low end of a bucket takes 128-token tiles with the same split
+  auto finish = [T](mlora_tile_config c) {
+    if (c.bm_shrink == 256 && (T + 255) / 256 * c.ksplit < 224) c.bm_shrink = 128;
+    return c;
+  };
   for (int i = 0; i < N_MEMO; ++i)
     if (memo[i].valid && memo[i].tb == tb && memo[i].rb == rb && memo[i].hidden == hidden && memo[i].ab == ab)
-      return memo[i].cfg;
+      return finish(memo[i].cfg);
   mlora_tile_config c;
   // the rule for shapes without an entry looks at T and A themselves, not at their buckets: not remembered
   // an adapter bucket without entries takes those of the next larger measured one, else of the next smaller
@@ -103,7 +109,7 @@ mlora_tile_config tile_lookup(int64_t T, int64_t max_rank, int64_t hidden, int64
   if (!found) return tile_fallback(T, max_rank, hidden, A);
   memo[next] = Memo{tb, rb, hidden, ab, c, true};
   next = (next + 1) % N_MEMO;
-  return c;
+  return finish(c);
 }
 
 // the entry of the shape's buckets (of the nearest measured width, if this one has none); false: no entry
