@@ -158,6 +158,8 @@ TABLE_CASES = [
     (11008, 300, 16, 1), (11008, 2000, 64, 1), (8192, 120, 32, 1), (2048, 1300, 16, 1), (28672, 400, 16, 1),
     (4096, 100, 16, 100), (4096, 400, 32, 32), (4096, 1500, 16, 100), (4096, 2000, 64, 32), (11008, 500, 64, 8),
     (4096, 300, 16, 500),
+    # 256-token shrink tiles (the table's choice for 16384 single-adapter tokens) and the 8192-token bucket
+    (4096, 16384, 64, 1), (4096, 16000, 32, 1), (4096, 9000, 64, 1), (4096, 8000, 64, 8), (11008, 6000, 16, 32),
 ]
 
 
