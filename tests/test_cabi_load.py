@@ -116,8 +116,8 @@ def test_tile_table_lookup_and_fallback():
     assert fb.bm_shrink == 128 and fb.ksplit >= 1 and not fb.reduce_in_expand
     fb = tt.fallback(300, 64, 4096, 200)            # decode-like -> direct 16-token tiles, expand sums the chunks
     assert fb.bm_shrink == 16 and fb.reduce_in_expand
-    assert tt.key(300, 16, 4096, 64) == "512:16:4096:128" and tt.key(600, 16, 4096, 64) == "1024:16:4096:128"
-    assert tt.key(300, 24, 4096, 64) == "512:32:4096:128" and tt.key(1, 8, 4096, 1) == "8:16:4096:1"
+    assert tt.key(300, 16, 4096, 64) == "512:16:4096:64" and tt.key(600, 16, 4096, 100) == "1024:16:4096:128"
+    assert tt.key(300, 24, 4096, 65) == "512:32:4096:128" and tt.key(1, 8, 4096, 1) == "8:16:4096:1"
     for rank in (8, 40, 128):                       # every table entry is a configuration the kernels take
         for T in (1, 300, 5000, 100000):
             c = tt.lookup(T, rank, 4096, 16)

@@ -25,7 +25,7 @@ const Entry kTable[] = {
 constexpr int kEntries = (int)(sizeof(kTable) / sizeof(kTable[0]));
 
 const int64_t kTokenBuckets[] = {8, 64, 128, 256, 512, 1024, 2048, 4096, 8192, 16384, (int64_t)1 << 22};
-const int64_t kAdapterBuckets[] = {1, 8, 32, 128, 8192};
+const int64_t kAdapterBuckets[] = {1, 8, 32, 64, 128, 8192};
 const int64_t kRankBuckets[] = {16, 32, 64, 128};
 
 template <int N>

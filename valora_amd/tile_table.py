@@ -20,7 +20,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 TABLE_PATH = os.path.join(_HERE, "tile_table.json")
 
 TOKEN_BUCKETS = (8, 64, 128, 256, 512, 1024, 2048, 4096, 8192, 16384, 1 << 22)
-ADAPTER_BUCKETS = (1, 8, 32, 128, 8192)
+ADAPTER_BUCKETS = (1, 8, 32, 64, 128, 8192)
 RANK_BUCKETS = (16, 32, 64, 128)
 
 

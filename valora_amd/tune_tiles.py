@@ -192,7 +192,7 @@ def main():
     ap.add_argument("--overwrite", action="store_true")
     ap.add_argument("--hidden", type=int, nargs="+", default=[4096])
     ap.add_argument("--tokens", type=int, nargs="+", default=[8, 64, 128, 256, 512, 1024, 2048, 4096, 8192, 16384])
-    ap.add_argument("--adapters", type=int, nargs="+", default=[8, 32, 128])
+    ap.add_argument("--adapters", type=int, nargs="+", default=[1, 8, 32, 64, 128])
     ap.add_argument("--ranks", type=int, nargs="+", default=list(tt.RANK_BUCKETS))
     ap.add_argument("--out", default=tt.TABLE_PATH)
     ap.add_argument("--one-launch", action="store_true",
