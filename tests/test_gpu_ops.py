@@ -41,6 +41,8 @@ def _case(seed, T, h_in, h_out, ranks, dtype, paged=True, id_style="random", sca
     (50, 11008, (64, 8), "runs"),
     (200, 768, (128, 64, 8), "random"),      # rank 128
     (90, 2048, (8, 16, 32), "holes"),        # ids outside [0, A): rows must stay untouched
+    (256, 4096, (16,) * 200, "random"),      # more adapters than the tile table has a bucket for
+    (3000, 1024, (64,), "random"),           # one adapter for the whole batch
 ])
 def test_dispatch_bgmv_shrink_and_expand(dev, dtype, T, h, ranks, ids_style):
     from valora_amd.kernels import dispatch_bgmv

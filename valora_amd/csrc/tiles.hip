@@ -156,11 +156,11 @@ int tile_ksplit_for(int64_t T, int64_t max_rank, int64_t hidden, int64_t A, int 
 
 // the largest split-K factor any width's entry of this shape asks for (workspace sizing)
 int tile_max_ksplit(int64_t T, int64_t max_rank, int64_t A) {
-  const int64_t tb = bucket(T, kTokenBuckets), rb = bucket(max_rank, kRankBuckets), ab = bucket(A, kAdapterBuckets);
+  // every adapter bucket counts: a bucket without entries of its own is served from a neighbouring one
+  const int64_t tb = bucket(T, kTokenBuckets), rb = bucket(max_rank, kRankBuckets);
   int ks = tile_fallback(T, max_rank, (int64_t)1 << 16, A).ksplit;
   for (int i = 0; i < kEntries; ++i)
-    if (kTable[i].tokens == tb && kTable[i].rank == rb && kTable[i].adapters == ab && kTable[i].ksplit > ks)
-      ks = kTable[i].ksplit;
+    if (kTable[i].tokens == tb && kTable[i].rank == rb && kTable[i].ksplit > ks) ks = kTable[i].ksplit;
   return ks;
 }
 
