@@ -506,6 +506,48 @@ def bench_single_adapter_vs_gemm(torch, W, LoraPlan, dev, use_graph, reps):
     return out
 
 
+def bench_tile_edge(torch, W, LoraPlan, dev, kb, vb, xs, ys, use_graph, n_draws=200, n_layers=8):
+    """The headline shape over `n_draws` seeded Zipf(0.6) draws of its per-token adapter ids (256 tokens, 64 rank-16
+    adapters, same pools, x and y as the headline): the device holds the one-launch grid of 64 tiles of up to 16 tokens
+    at once, and a draw has 55-66 of them.  Per draw: the one-launch op and, on the same operands, the two-launch op
+    with the same split (bit-identical results); reported: median, p99 and max of the one-launch time and the worst
+    ratio to the same draw's two launches."""
+    pool_idx = None
+    rows = []
+    for seed in range(n_draws):
+        g = torch.Generator().manual_seed(7000 + seed)
+        ids = W.zipf_ids(64, 256, 0.6, g)
+        cnt = torch.bincount(ids, minlength=64)
+        n_tiles = int(((cnt + 15) // 16).sum())
+        idd = ids.to(dev)
+        if pool_idx is None:
+            pool_idx = W.config2().to(dev).targets[0].pool
+        p = pool_idx
+        us = []
+        for kw in (dict(one_launch=True, ksplit=4),
+                   dict(one_launch=False, bm_shrink=16, bm_expand=16, ksplit=4, reduce_in_expand=True)):
+            plan = LoraPlan(idd, p.a_start, p.a_len, 16, hidden=4096, **kw)
+
+            def run():
+                for l in range(n_layers):
+                    plan.apply(ys[l], xs[l], kb[l], vb[l], p.a_start, p.a_len, p.a_loc, 0, p.a_scaling)
+
+            us.append(time_graph(torch, run, 10, 2, use_graph)[0] * 1e3 / n_layers)
+        rows.append((n_tiles, us[0], us[1]))
+    one = sorted(r[1] for r in rows)
+    by_tiles = {}
+    for n, a, b in rows:
+        by_tiles.setdefault(n, []).append((a, b))
+    return {"draws": n_draws, "layers_per_timing": n_layers,
+            "one_launch_us": {"median": round(one[len(one) // 2], 2), "p99": round(one[int(0.99 * (len(one) - 1))], 2),
+                              "max": round(one[-1], 2)},
+            "two_launch_us_median": round(sorted(r[2] for r in rows)[len(rows) // 2], 2),
+            "worst_one_over_two_of_a_draw": round(max(a / b for _, a, b in rows), 3),
+            "by_tile_count": {str(n): {"draws": len(v), "one_launch_us": round(sum(a for a, _ in v) / len(v), 2),
+                                       "two_launch_us": round(sum(b for _, b in v) / len(v), 2)}
+                              for n, v in sorted(by_tiles.items())}}
+
+
 def bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, reps, no_step5):
     """Legs beside the headline, all on the config-2 decode shape with the same rotation over `L` layers'
     buffers: a whole attention block's LoRA work per layer, and the same shrink + expand pair reached through
@@ -607,6 +649,10 @@ def bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, r
     out["dropin_pair_is"] = ("shrink + expand of the config-2 op through the reference's own entry points (two calls per "
                              "layer, torch binding -> one C-ABI call each with the cached plan of the batch); graph = HIP "
                              "graph replay, eager = launched from Python call by call (events / host wall clock)")
+    try:
+        out["tile_edge"] = bench_tile_edge(torch, W, LoraPlan, dev, kb, vb, xs, ys, use_graph)
+    except Exception as exc:    # the headline does not depend on this leg
+        out["tile_edge"] = {"error": f"{type(exc).__name__}: {exc}"}
     try:
         out["byte_heavy_decode"] = bench_byte_heavy_decode(torch, W, LoraPlan, dev, use_graph, reps)
     except Exception as exc:    # the headline does not depend on this leg

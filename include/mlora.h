@@ -45,15 +45,17 @@ enum {
                                  with the same ksplit.                                            */
   MLORA_ONE_LAUNCH = 2,       /* mlora_lora_apply / mlora_lora_apply_multi only: shrink and expand are
                                  work items of ONE grid; an expand item requests its B and y operands,
-                                 then waits (bounded) for its tile's K-chunk partials and computes them
-                                 itself if they do not come.  For decode-like batches: needs a plan cut
-                                 with bm_shrink = bm_expand = 16 and max_rank <= 64; ksplit is raised to
-                                 2 if smaller and cut so that ksplit * n_targets <= 16; scratch of
-                                 mlora_one_launch_scratch_bytes().  A batch whose grid the device cannot
-                                 hold all at once is run as two launches instead.  Bit-identical to the
-                                 two-launch op with
-                                 MLORA_REDUCE_IN_EXPAND and the same ksplit.  Launches that share a plan
-                                 must not overlap in time.                                        */
+                                 then waits (bounded: 30 us) for its tile's K-chunk partials and computes
+                                 them itself if they do not come.  For decode-like batches: needs a plan
+                                 cut with bm_shrink = bm_expand = 16 and max_rank <= 64; ksplit is raised
+                                 to 2 if smaller and cut so that ksplit * n_targets <= 16; scratch of
+                                 mlora_one_launch_scratch_bytes(), 128-byte aligned (the partials are
+                                 handed over in cache lines that belong to one tile each; a scratch
+                                 buffer aligned to less, an empty index or an empty pool make the call
+                                 run as two launches).  Any batch size: items the device cannot hold
+                                 from the start take part in the hand-off like the others.
+                                 Bit-identical to the two-launch op with MLORA_REDUCE_IN_EXPAND and the
+                                 same ksplit.  Launches that share a plan must not overlap in time.  */
   MLORA_ONE_LAUNCH_NO_WAIT = 4, /* with MLORA_ONE_LAUNCH: expand items do not wait at all and always
                                  compute their tile's partials themselves (the give-up path made
                                  testable; same results, slower)                                  */

@@ -2,10 +2,10 @@
 
 Its contract is "bit-identical to the two-launch op with the same ksplit whose expand sums the K chunks", on
 every path an item can take: partials handed over by the shrink items, partials recomputed because the wait
-was given up (forced from the host with a poll bound of zero -- no kernel is ever made to wait or hang), items
-the device cannot hold from the start, several targets in one call, and -- the part a single call cannot
-show -- launch after launch on one plan, where a stamp left behind by the previous launch must never be taken
-for a fresh one."""
+was given up (forced from the host with a wait bound of zero -- no kernel is ever made to wait or hang), items
+the device cannot hold from the start (they take part in the hand-off like the others), several targets in one
+call, and -- the part a single call cannot show -- launch after launch on one plan, where a stamp left behind by
+the previous launch must never be taken for a fresh one."""
 import random
 
 import pytest
@@ -172,8 +172,8 @@ def test_one_launch_random_shapes(dev, seed):
 @pytest.mark.parametrize("ks", [4, 5])
 def test_items_the_device_cannot_hold_from_the_start(dev, ks):
     """64 tiles of one token each at 4096 -> 4096: with 5 K chunks the grid is larger than what the device
-    holds at once, so the last tiles' expand items start late by construction and must not trust stamps;
-    with 4 it just fits.  Either way the result is the two-launch op's."""
+    holds at once, so the last tiles' expand items start late by construction; with 4 it just fits.  Either way
+    the result is the two-launch op's."""
     dtype = torch.float16
     g = torch.Generator().manual_seed(77)
     A, T, h = 64, 64, 4096
@@ -196,10 +196,55 @@ def test_items_the_device_cannot_hold_from_the_start(dev, ks):
     assert_parity(a.cpu(), ref, "late items")
 
 
-def test_one_launch_request_on_a_large_batch_runs_as_two_launches(dev):
-    """A batch whose grid is far larger than the device is not run through the one-launch kernel (the library
-    decides per call); the request is honoured with the same bits."""
-    w = W.config3(hidden=512, mlp=1024, len_div=2, n_decode=64, targets=("q",))
+@pytest.mark.parametrize("n_tiles", [64, 65, 66, 76])
+def test_batches_at_the_edge_of_what_the_device_holds(dev, n_tiles):
+    """The benchmark's decode shape (256 tokens, 64 rank-16 adapters, 4096 -> 4096, 4 K chunks) with adapter counts
+    made so that the batch has exactly `n_tiles` tiles of up to 16 tokens: 64 fill the device, 65 and 66 are what
+    a Zipf(0.6) draw gives now and then, 76 is the most this shape can have.  The tiles beyond the device's
+    capacity start late and use the hand-off like the others; layer after layer on one plan, results equal the
+    two-launch op's bit for bit."""
+    dtype = torch.float16
+    A, T, h = 64, 256, 4096
+    extra = n_tiles - 64                      # adapters that own 17 tokens: two tiles each
+    cnt = [17] * extra + [1] * (A - extra)
+    spare = T - sum(cnt)
+    k = extra
+    while spare > 0:                          # hand the rest out without crossing another multiple of 16
+        add = min(spare, 15)
+        cnt[k] += add
+        spare -= add
+        k += 1
+    assert sum(cnt) == T and sum((c + 15) // 16 for c in cnt) == n_tiles
+    g = torch.Generator().manual_seed(900 + n_tiles)
+    ids = torch.repeat_interleave(torch.arange(A), torch.tensor(cnt))[torch.randperm(T, generator=g)]
+    pool = W.make_pool([16] * A, h, h, dtype, g, True, std=0.05)
+    pd = pool.to(dev)
+    idx = (pd.a_start, pd.a_len, pd.a_loc)
+    one = LoraPlan(ids.to(dev), pd.a_start, pd.a_len, 16, hidden=h, one_launch=True, ksplit=4)
+    two = LoraPlan(ids.to(dev), pd.a_start, pd.a_len, 16, hidden=h, one_launch=False, bm_shrink=16, bm_expand=16,
+                   ksplit=4, reduce_in_expand=True)
+    assert one.header()["n_tiles_expand"] == n_tiles
+    gd = torch.Generator(device=dev).manual_seed(n_tiles)
+    xs = [torch.randn(T, h, generator=gd, device=dev).to(dtype) for _ in range(6)]
+    y0 = [torch.randn(T, h, generator=gd, device=dev).to(dtype) for _ in range(6)]
+    for rep in range(2):
+        got, want = [y.clone() for y in y0], [y.clone() for y in y0]
+        for l in range(6):
+            one.apply(got[l], xs[l], pd.key_buffer, pd.value_buffer, *idx, l % 4, pd.a_scaling)
+            two.apply(want[l], xs[l], pd.key_buffer, pd.value_buffer, *idx, l % 4, pd.a_scaling)
+        torch.cuda.synchronize()
+        for l in range(6):
+            assert torch.equal(got[l], want[l]), f"{n_tiles} tiles, repetition {rep}, layer {l}"
+    ref = O.lora_op(y0[0].cpu(), xs[0].cpu(), pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc,
+                    ids, 0, pool.a_scaling)
+    assert_parity(got[0].cpu(), ref, f"{n_tiles} tiles vs oracle")
+
+
+def test_a_batch_several_times_the_device_runs_as_one_launch(dev):
+    """A mixed batch whose one-launch grid is many times what the device holds (and three targets on top): the
+    items run as a pipeline of shrink items followed by expand items, all through the hand-off; same bits as
+    two launches."""
+    w = W.config3(hidden=512, mlp=1024, len_div=2, n_decode=64, targets=("q", "k", "v"))
     wd = w.to(dev)
     t = wd.target("q"); p = t.pool
     R = max(p.ranks)
@@ -208,6 +253,13 @@ def test_one_launch_request_on_a_large_batch_runs_as_two_launches(dev):
     one.apply(a, wd.x[512], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
     two.apply(b, wd.x[512], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
     assert torch.equal(a, b)
+    for rep in range(2):
+        ya = [wd.y0[n].clone() for n in ("q", "k", "v")]
+        yb = [wd.y0[n].clone() for n in ("q", "k", "v")]
+        for plan, ys in ((one, ya), (two, yb)):
+            plan.apply_multi(ys, wd.x[512], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, [0, 1, 2], p.a_scaling)
+        for u, v in zip(ya, yb):
+            assert torch.equal(u, v), f"three targets, repetition {rep}"
 
 
 def test_one_launch_op_and_in_launch_split_k_sum_share_a_plan(dev):

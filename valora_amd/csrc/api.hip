@@ -29,15 +29,16 @@ int check_launch(const char *what) {
 int expand_bn();
 int decode_bn(int max_rank);   // output columns per expand item of the one-launch op
 
-// Polls of a tile's "ready" word before an expand item of the one-launch op stops waiting and computes the
-// tile's partials itself.  A poll is one memory round trip plus a short sleep (about a microsecond), the shrink
-// items it waits for run for a few microseconds: the bound is far above anything a healthy launch needs and
-// only limits how long a workgroup can wait when its producers have not been scheduled.
-constexpr int ONE_LAUNCH_SPIN_LIMIT = 1024;
+// How long an expand item of the one-launch op waits for its tile's shrink items before it computes the tile's
+// partials itself, in ticks of the device's 100 MHz clock: 30 us.  The shrink items are started before the expand
+// items that wait for them and run for a few microseconds, so a healthy launch never gets near the bound; it only
+// limits how long a workgroup holds its slot when the producers are held up (a device shared with other work).
+constexpr int ONE_LAUNCH_WAIT_TICKS = 3000;
 
 namespace {
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool aligned128(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 127u) == 0; }
 
 const char *dtype_name(mlora_dtype dt) { return dt == MLORA_F16 ? "Half" : "BFloat16"; }
 
@@ -123,7 +124,9 @@ PoolDev pool_dev(const mlora_pool *p) {
 // sum to the expand).
 void set_reduce_here(ShrinkArgs &a, const mlora_plan *plan, const PlanLayout &L, int64_t max_rank, int flags) {
   const int64_t tile_bytes = (int64_t)a.ksplit * plan->bm_shrink * partial_stride_lines(max_rank) * 4;
-  const bool small = plan->bm_shrink <= 64 && tile_bytes <= 65536 && plan->T <= 4096;
+  // (the partials' rows must really begin on 128-byte lines: a scratch buffer that is only 16-byte aligned keeps the
+  // reduce launch)
+  const bool small = plan->bm_shrink <= 64 && tile_bytes <= 65536 && plan->T <= 4096 && aligned128(a.partial);
   a.reduce_here = (small && a.ksplit > 1 && !a.partial_only) ? ((flags & MLORA_SHRINK_RECOMPUTE) ? 2 : 1) : 0;
   a.prp = (int)partial_stride_lines(max_rank);
   a.n_tiles = (int)tiles_upper(plan->T, plan->n_adapters, plan->bm_shrink);
@@ -418,19 +421,12 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
     if (ksplit < 2) ksplit = 2;   // the hand-off carries fp32 K-chunk partials
     if (ksplit * n_targets > DECODE_MAX_PRODUCERS) ksplit = DECODE_MAX_PRODUCERS / n_targets;
   }
-  // The one-launch op is for grids the device holds (nearly) all at once: an item that starts late cannot
-  // take its tile's partials from the shrink items and computes them itself.  The grid is sized with an upper
-  // bound of the tile count, so some slack is allowed for workgroups that find no tile; a larger batch runs as
-  // two launches with the same ksplit, which gives the same bits.
-  bool one_launch_fits = false;
-  int decode_resident = 0;
-  if (one_launch) {
-    const int64_t groups8 = (tiles_upper(T, plan->n_adapters, 16) + 7) / 8 * 8;
-    const int64_t items = groups8 * ksplit * n_targets + groups8 * ((h_out + decode_bn((int)max_rank) - 1) / decode_bn((int)max_rank)) * n_targets;
-    decode_resident = decode_resident_workgroups((int)max_rank, dtype);
-    one_launch_fits = (flags & MLORA_ONE_LAUNCH_NO_WAIT) || (decode_resident > 0 && items * 4 <= (int64_t)decode_resident * 5);
-  }
-  const bool use_decode = one_launch && one_launch_fits;
+  // The one-launch op hands the K-chunk partials over inside the launch, through lines of the scratch buffer that
+  // belong to one tile each (128-byte aligned), and its expand items read element 0 of the index and of every
+  // target's pool where they have nothing to fetch: a call that cannot offer that runs as two launches with the
+  // same ksplit, which gives the same bits.
+  bool use_decode = one_launch && aligned128(scratch) && pool_a->a_loc_len > 0 && pool_a->w_rows > 0;
+  for (int i = 0; use_decode && i < n_targets; ++i) use_decode = targets[i].w_b_rows > 0;
   if (ksplit < 1 || ksplit > 64) return fail(MLORA_ERR_INVALID, "lora_apply_multi: ksplit=%d outside [1,64]", ksplit);
   const size_t per_target = scratch_bytes(T, max_rank, ksplit);
   const size_t scratch_need = use_decode ? mlora_one_launch_scratch_bytes(T, plan->n_adapters, max_rank, ksplit, n_targets)
@@ -516,10 +512,7 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
     d.e.n_ochunks = (int)((h_out + decode_bn((int)max_rank) - 1) / decode_bn((int)max_rank));
     d.n_producers = ksplit * n_targets;
     d.n_consumers = d.e.n_ochunks * n_targets;
-    d.groups_per_chunk = decode_resident / (8 * (d.n_producers + d.n_consumers));
-    if (d.groups_per_chunk < 1) d.groups_per_chunk = 1;
-    d.spin_limit = (flags & MLORA_ONE_LAUNCH_NO_WAIT) ? 0 : ONE_LAUNCH_SPIN_LIMIT;
-    d.resident = decode_resident;
+    d.spin_limit = (flags & MLORA_ONE_LAUNCH_NO_WAIT) ? 0 : ONE_LAUNCH_WAIT_TICKS;
     return launch_decode((hipStream_t)stream, d, (int)max_rank, dtype);
   }
   return launch_expand((hipStream_t)stream, e, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand),

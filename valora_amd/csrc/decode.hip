@@ -24,14 +24,24 @@
 //     workgroups;
 //   * the stamps are polled on the scalar path (scalar load that skips the scalar cache): a wave gets its
 //     vector-memory results strictly in order, so a vector poll would sit behind the B and y loads;
-//   * what tells a fresh stamp from one an earlier launch left behind is the tile's `done` word: every shrink
-//     item adds 1 to it when it has finished (device scope, nobody waits for the answer), and every item reads
-//     it when it starts and uses the value as the launch's tag.  All items that start before the tile's first
-//     shrink item finishes (microseconds later) read the same value, and it differs from every earlier
-//     launch's.  An item that starts later reads another value and matches nothing: correct, and slow.
-//     Therefore the items the device cannot hold from the start do not use the hand-off at all (see
-//     decode_kernel), and the host only picks this kernel for grids that (nearly) fit the device.
-//     Nothing is ever reset, so there is no moment at which a late writer could leave a stale "ready".
+//   * what tells a fresh stamp from one an earlier launch left behind is the launch's tag, which every item
+//     derives from the tile's `done` word as it finds it when it starts: tag = word / DECODE_LAUNCH_WEIGHT.  Every
+//     launch moves the word on by exactly that weight, whatever its numbers of shrink and expand items: each
+//     shrink item adds 1 when it has finished, and the tile's LAST expand item (highest id) adds the rest at its
+//     very end (device scope, nobody waits for the answer).  Launches on a plan do not overlap, so in launch
+//     number n no item can read less than n * weight: a tag is never too low, and a stamp an earlier launch left
+//     behind is never taken for a fresh one.  An item would read (n + 1) * weight, and match nothing, only if it
+//     read the word after the tile's last expand item had ENDED.  The hardware starts workgroups in id order and
+//     the read is an item's first instruction, so that takes an item whose first load is outlived by the whole
+//     life of an item started after it; it would wait out its bound and compute the partials itself: slow, and
+//     still correct.  Items that start late (a grid larger than the device holds, a device shared with another
+//     stream) therefore take part in the hand-off like all others.  Nothing is ever reset, so there is no moment
+//     at which a late writer could leave a stale "ready", and replays of a HIP graph (frozen arguments) need
+//     nothing from the host.  (Every expand item adding its own share would make the bound on the word exact,
+//     and costs 0.4 us on a 9.7 us op: the device-scope acknowledgements of 512 workgroups at the end of the
+//     launch.)
+//   * all shrink items have lower ids than all expand items, so by the time an expand item runs, every producer
+//     it waits for has at least been started.
 //   * a tile's partials occupy whole 128-byte lines of their own, so no line is fetched before the tile is
 //     ready (a line shared with a neighbour tile could sit stale in a compute unit's L1).
 // Chunks are summed in index order, the same order as the two-launch path: results are bit-identical to it.
@@ -61,60 +71,62 @@ __device__ __forceinline__ void add_device(uint32_t *p, uint32_t v) {
 // glc skips the scalar cache, and its answer does not queue behind the wave's outstanding vector loads (the B
 // fragments and y rows requested just before), which come back strictly in order.
 typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
-__device__ __forceinline__ bool stamps_match(const uint32_t *stamps, int n, uint32_t want) {
+// 1: all n stamps carry `want`; 2: one of them carries this launch's tag with another XCD's id, i.e. that producer
+// ran where its partial cannot be read from here, and waiting longer is pointless; 0: not yet.
+__device__ __forceinline__ int stamps_state(const uint32_t *stamps, int n, uint32_t want) {
   u32x16 v;
   asm volatile("s_load_dwordx16 %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(stamps) : "memory");
-  bool ok = true;
+  // d = stamp ^ want is 0 for a match and 1..15 for this launch's tag with another XCD id (branch-free scalar code)
+  uint32_t any_diff = 0u, least = 0xffffffffu;
 #pragma unroll
-  for (int i = 0; i < DECODE_MAX_PRODUCERS; ++i) ok = ok && (i >= n || v[i] == want);
-  return ok;
+  for (int i = 0; i < DECODE_MAX_PRODUCERS; ++i) {
+    const uint32_t d = i < n ? (v[i] ^ want) : 0u;
+    any_diff |= d;
+    const uint32_t u = d - 1u;   // 0 -> 0xffffffff
+    least = u < least ? u : least;
+  }
+  return any_diff == 0u ? 1 : least < 15u ? 2 : 0;
 }
 // workgroup barrier that orders LDS traffic only: outstanding global loads stay in flight across it
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-__device__ __forceinline__ uint32_t stamp_of(uint32_t tag, uint32_t xcd) { return ((tag + 1u) << 4) | xcd; }
+// the launch's tag from the tile's `done` word as an item found it (see the head of this file), and the stamp a
+// shrink item of that launch leaves when it runs on XCD `xcd` (never 0, the value the plan kernel leaves)
+__device__ __forceinline__ uint32_t stamp_of(uint32_t done0, uint32_t xcd) {
+  return (((done0 >> DECODE_TAG_SHIFT) + 1u) << 4) | xcd;
+}
 
-// item id -> (role, tile, item of the tile).  A group is 8 consecutive tiles, a chunk as many groups as the
-// device holds at once.  Ids run chunk by chunk: first the chunk's shrink items, then its expand items, each as
-// (group, item, tile within the group) with the tile as the fast index, so the tile index mod 8 equals the id
-// mod 8 and the shrink items of the resident part of the grid are the first to be started.  The grid is sized
-// with an upper bound of the tile count; the tiles that do not exist are the last ones, so their items have
-// the highest ids of their chunk.
+// item id -> (role, tile, item of the tile).  A group is 8 consecutive tiles.  Ids run: the shrink items of all
+// groups, then the expand items of all groups, each as (group, item, tile within the group) with the tile as the
+// fast index, so the tile index mod 8 equals the id mod 8 (one XCD per tile) and every producer is started before
+// any consumer.  The grid is sized with an upper bound of the tile count; the tiles that do not exist are the
+// last ones of either section, and their workgroups leave at once (measured against a layout that puts them at
+// the end of the grid: equal on a batch that fits the device, 2 us faster on one that does not quite).
 struct ItemId {
   bool shrink;
   int tile, item;
 };
-__device__ __forceinline__ ItemId item_of(int n_producers, int n_consumers, int groups_per_chunk, int id) {
+__device__ __forceinline__ ItemId item_of(int n_producers, int n_consumers, int shrink_ids, int id) {
   ItemId it;
-  const int per_group = 8 * (n_producers + n_consumers);
-  const int per_chunk = groups_per_chunk * per_group;
-  const int chunk = id / per_chunk, local = id - chunk * per_chunk;
-  const int n_shrink = groups_per_chunk * 8 * n_producers;
-  it.shrink = local < n_shrink;
-  const int l2 = it.shrink ? local : local - n_shrink;
+  it.shrink = id < shrink_ids;
+  const int l2 = it.shrink ? id : id - shrink_ids;
   const int per = it.shrink ? n_producers : n_consumers;
   const int q8 = l2 >> 3, g = q8 / per;
   it.item = q8 - g * per;
-  it.tile = (chunk * groups_per_chunk + g) * 8 + (l2 & 7);
+  it.tile = g * 8 + (l2 & 7);
   return it;
 }
 
-// One workgroup = one work item.  The first `resident` workgroups are the ones the device holds from the start
-// (the hardware starts workgroups in id order); whatever has a higher id may start late, i.e. after shrink
-// items of its tile have finished and moved the tile's tag on.  Such an expand item does not look at stamps
-// at all but computes its tile's partials itself, and such a shrink item has nobody who would use its result
-// (a tile's expand items come after its shrink items) and does nothing.  With the ids running chunk by
-// chunk, these are the items of the tiles that do not exist, unless the batch is larger than the device.
-// 3 waves per SIMD = 3 workgroups per compute unit: an expand item keeps the B fragments and y rows of 512
-// columns in flight, a shrink item 8 K-steps of both operands.
+// One workgroup = one work item.  3 waves per SIMD = 3 workgroups per compute unit: an expand item keeps the B
+// fragments and y rows of 512 columns in flight, a shrink item 8 K-steps of both operands.
 // The leading scalar parameters repeat what the first dependent loads need (the tile records, the `done` words, the
 // id layout): the library is built with kernel-argument preloading, which hands the first 8 dwords of the
 // argument list to the wave in registers at launch, so the tile record can be requested without waiting for a load
 // of the argument block first (0.35 us of a 10.3 us op).
 template <typename T, int NB>
-__global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_base, const uint32_t *done_base, int h_n_producers,
-                                                        int h_n_consumers, int h_groups_per_chunk, int h_n_tiles,
-                                                        int h_resident, DecodeArgs a) {
+__global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_base, uint32_t *done_base, int h_n_producers,
+                                                        int h_n_consumers, int h_n_tiles, int h_shrink_ids,
+                                                        DecodeArgs a) {
   using Tr = Traits<T>;
   using vec8 = typename Tr::vec8;
   constexpr int DEC_CH = dec_ch(NB), DEC_BN = 256 * DEC_CH;   // chunks and outputs per expand item
@@ -129,15 +141,13 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
   __shared__ int32_t s_ready;
   float(*red)[NB * 256] = reinterpret_cast<float(*)[NB * 256]>(s_buf);
   const int id = (int)blockIdx.x;
-  const bool on_time = id < h_resident;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-  const ItemId it = item_of(h_n_producers, h_n_consumers, h_groups_per_chunk, id);
+  const ItemId it = item_of(h_n_producers, h_n_consumers, h_shrink_ids, id);
   const bool shrink_item = it.shrink;
   const int item = it.item, tile_idx = it.tile;
   if (tile_idx >= h_n_tiles) return;
-  if (shrink_item && !on_time) return;
   const int32_t *__restrict__ tile = tiles_base + (int64_t)tile_idx * TILE_WORDS;
 
   // ONE scalar round trip per shrink item before its vector loads: the tile record, the tile's `done` word and every
@@ -160,7 +170,7 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
     PoolDev pool = a.s.pool;
     int h_in = a.s.h_in, ksplit = a.s.ksplit, kchunk = a.s.kchunk;
     int sl0 = a.s.slots[0], sl1 = a.s.slots[1], sl2 = a.s.slots[2], sl3 = a.s.slots[3];
-    uint32_t *done = a.done;
+    uint32_t *done = done_base;
     asm volatile("" : "+s"(ad), "+s"(r), "+s"(pos0), "+s"(cnt), "+s"(astart), "+s"(done0), "+s"(rp), "+s"(n_producers),
                       "+s"(plan_words), "+s"(off_perm), "+s"(partial_base), "+s"(stamps_base), "+s"(x), "+s"(pool.w),
                       "+s"(pool.w_rows), "+s"(pool.a_loc), "+s"(pool.a_loc_len), "+s"(h_in), "+s"(ksplit), "+s"(kchunk),
@@ -173,7 +183,6 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
     partial_base = as_global(partial_base);
     stamps_base = as_global(stamps_base);
     const int32_t *__restrict__ perm = as_global(plan_words) + off_perm;
-    // the launch's tag: what the tile's `done` word holds while none of this launch's shrink items has finished
     const uint32_t want_stamp = stamp_of(done0, xcd_id());
     uint32_t *const stamps = stamps_base + (int64_t)tile_idx * DECODE_MAX_PRODUCERS;
     // a tile's partials: [target][K chunk][16 rows][rp] floats, whole lines of the tile's own
@@ -196,7 +205,7 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
       wait_vmcnt<0>();
       if (lane == 0) __hip_atomic_store(stamps + item, want_stamp, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     } else if (tid == 64) {
-      add_device(done + tile_idx, 1u);
+      add_device(done + tile_idx, 1u);   // this item's share of the launch's weight on the tile's `done` word
     }
     return;
   }
@@ -289,12 +298,19 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
       yv[c][h] = load16(yp[c][h]);
     }
   // ---- bounded wait for the tile's stamps (one wave polls on the scalar path; the workgroup follows its
-  //      verdict without draining its loads)
+  //      verdict without draining its loads).  The producers were started before this item and run for a few
+  //      microseconds; the bound (ticks of the 100 MHz clock, and a cap on the polls) only limits how long a
+  //      workgroup can hold its slot when they are held up, and a producer seen on another XCD ends the wait at once.
   if (wave == 0) {
     int ok = 0;
-    for (int it = 0; on_time && it < spin_limit; ++it) {
-      if (stamps_match(stamps, n_producers, want_stamp)) { ok = 1; break; }
-      __builtin_amdgcn_s_sleep(2);
+    if (spin_limit > 0) {
+      const uint64_t t0 = wall_clock64();
+      for (int it = 0; it < ONE_LAUNCH_MAX_POLLS; ++it) {
+        const int st = stamps_state(stamps, n_producers, want_stamp);
+        if (st == 1) ok = 1;
+        if (st != 0 || wall_clock64() - t0 > (uint64_t)spin_limit) break;
+        __builtin_amdgcn_s_sleep(2);
+      }
     }
     if (lane == 0) s_ready = ok;
   }
@@ -391,15 +407,16 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
       __builtin_amdgcn_wave_barrier();
     }
   }
-
+  // the tile's last expand item tops the tile's `done` word up to the launch's weight
+  if (tid == 0 && item == h_n_consumers - 1) add_device(done_base + tile_idx, DECODE_LAUNCH_WEIGHT - (uint32_t)n_producers);
 }
 
 template <typename T>
-int launch_decode_t(hipStream_t st, const DecodeArgs &a, int nb, dim3 grid) {
+int launch_decode_t(hipStream_t st, const DecodeArgs &a, int nb, dim3 grid, int shrink_ids) {
   switch (nb) {
-    case 1: hipLaunchKernelGGL((decode_kernel<T, 1>), grid, dim3(256), 0, st, a.s.plan + a.e.off_tiles, (const uint32_t *)a.done, a.n_producers, a.n_consumers, a.groups_per_chunk, a.n_tiles, a.resident, a); break;
-    case 2: hipLaunchKernelGGL((decode_kernel<T, 2>), grid, dim3(256), 0, st, a.s.plan + a.e.off_tiles, (const uint32_t *)a.done, a.n_producers, a.n_consumers, a.groups_per_chunk, a.n_tiles, a.resident, a); break;
-    case 4: hipLaunchKernelGGL((decode_kernel<T, 4>), grid, dim3(256), 0, st, a.s.plan + a.e.off_tiles, (const uint32_t *)a.done, a.n_producers, a.n_consumers, a.groups_per_chunk, a.n_tiles, a.resident, a); break;
+    case 1: hipLaunchKernelGGL((decode_kernel<T, 1>), grid, dim3(256), 0, st, a.s.plan + a.e.off_tiles, a.done, a.n_producers, a.n_consumers, a.n_tiles, shrink_ids, a); break;
+    case 2: hipLaunchKernelGGL((decode_kernel<T, 2>), grid, dim3(256), 0, st, a.s.plan + a.e.off_tiles, a.done, a.n_producers, a.n_consumers, a.n_tiles, shrink_ids, a); break;
+    case 4: hipLaunchKernelGGL((decode_kernel<T, 4>), grid, dim3(256), 0, st, a.s.plan + a.e.off_tiles, a.done, a.n_producers, a.n_consumers, a.n_tiles, shrink_ids, a); break;
     default: return fail(MLORA_ERR_NO_KERNEL, "one-launch op: ranks above 64 use the two-launch path");
   }
   return check_launch("decode_kernel");
@@ -408,32 +425,6 @@ int launch_decode_t(hipStream_t st, const DecodeArgs &a, int nb, dim3 grid) {
 }  // namespace
 
 int decode_bn(int max_rank) { return 256 * dec_ch(dec_nb(max_rank)); }
-
-// How many workgroups of decode_kernel the current device can hold at the same time (0 if the runtime cannot
-// tell).  The one-launch op is only used for grids that fit: an item that starts after its tile's shrink
-// items have finished falls back to computing the partials itself, which is correct and slow.
-int decode_resident_workgroups(int max_rank, mlora_dtype dt) {
-  int nb = (max_rank + 15) / 16;
-  nb = nb <= 1 ? 0 : nb <= 2 ? 1 : 2;
-  static int cached[64][2][3];   // [device][dtype][rank class], 0 = not asked yet
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-  int &slot = cached[dev][dt == MLORA_F16 ? 0 : 1][nb];
-  if (slot > 0) return slot;
-  const void *fn = nullptr;
-  if (dt == MLORA_F16)
-    fn = nb == 0 ? (const void *)decode_kernel<_Float16, 1> : nb == 1 ? (const void *)decode_kernel<_Float16, 2>
-                                                                      : (const void *)decode_kernel<_Float16, 4>;
-  else
-    fn = nb == 0 ? (const void *)decode_kernel<__bf16, 1> : nb == 1 ? (const void *)decode_kernel<__bf16, 2>
-                                                                    : (const void *)decode_kernel<__bf16, 4>;
-  int per_cu = 0, cus = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 256, 0) != hipSuccess) return 0;
-  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-  if (per_cu <= 0 || cus <= 0) return 0;
-  slot = per_cu * cus;
-  return slot;
-}
 
 // floats of scratch the one-launch op needs for its partials: [tile][target][K chunk][16][rp]
 size_t decode_partial_floats(int64_t n_tiles, int n_targets, int ksplit, int64_t rp) {
@@ -446,13 +437,13 @@ int launch_decode(hipStream_t st, const DecodeArgs &a, int max_rank, mlora_dtype
   if (a.n_tiles <= 0) return MLORA_OK;
   if (a.n_producers > DECODE_MAX_PRODUCERS)
     return fail(MLORA_ERR_NO_KERNEL, "one-launch op: ksplit * targets = %d exceeds %d", a.n_producers, DECODE_MAX_PRODUCERS);
-  // whole chunks: the ids of a chunk that has fewer groups than the others still span a whole chunk
   const int64_t groups = (a.n_tiles + 7) / 8;
-  const int64_t chunks = (groups + a.groups_per_chunk - 1) / a.groups_per_chunk;
-  const int64_t total = chunks * a.groups_per_chunk * 8 * ((int64_t)a.n_producers + a.n_consumers);
+  const int64_t shrink_ids = groups * 8 * a.n_producers;
+  const int64_t total = shrink_ids + groups * 8 * a.n_consumers;
   if (total > 0x7fffffff) return fail(MLORA_ERR_NO_KERNEL, "one-launch op: grid too large");
   dim3 grid((unsigned)total);
-  return dt == MLORA_F16 ? launch_decode_t<_Float16>(st, a, nb, grid) : launch_decode_t<__bf16>(st, a, nb, grid);
+  return dt == MLORA_F16 ? launch_decode_t<_Float16>(st, a, nb, grid, (int)shrink_ids)
+                         : launch_decode_t<__bf16>(st, a, nb, grid, (int)shrink_ids);
 }
 
 }  // namespace mlora

@@ -16,8 +16,8 @@ namespace mlora {
 //             inside a group); positions >= hdr[H_NACTIVE] are unused
 // padapter[p] adapter of position p;  prank[p] its rank
 // tile        {adapter, rank, first position, token count, a_start[adapter], 0, 0, 0}
-// done, stamps  the hand-off words of the one-launch op (csrc/decode.hip): per tile a count of the shrink items
-//             that have finished on this plan, and one stamp per shrink item; zeroed by the plan kernel
+// done, stamps  the hand-off words of the one-launch op (csrc/decode.hip): per tile a word that numbers the launches
+//             on this plan, and one stamp per shrink item; zeroed by the plan kernel
 // arrive      the arrival words of the shrink's own split-K sum (csrc/shrink.hip): one 64-bit word per tile and
 //             target, zeroed by the plan kernel and back at zero after every launch
 constexpr int HDR_WORDS = 32;
@@ -25,15 +25,18 @@ constexpr int TILE_WORDS = 8;
 constexpr int32_t PLAN_MAGIC = 0x4d4c5241;
 enum Hdr {
   H_MAGIC = 0, H_T = 1, H_NADAPTERS = 2, H_NTILES_S = 3, H_NTILES_E = 4, H_NGROUPS = 5,
-  H_MAXRANK = 6, H_ERR = 7, H_BM_S = 8, H_BM_E = 9, H_NACTIVE = 10
+  H_MAXRANK = 6, H_RESERVED = 7, H_BM_S = 8, H_BM_E = 9, H_NACTIVE = 10
 };
-// bits of hdr[H_ERR]
-enum PlanErr { PERR_START_OVERFLOW = 1 };
 
 constexpr int64_t MAX_ADAPTERS = 8192;   // per-wave histograms live in LDS
 constexpr int64_t MAX_TOKENS = 1 << 22;
 constexpr int MAX_RANK = 128;
 constexpr int DECODE_MAX_PRODUCERS = 16;   // shrink items per tile (K chunks x targets) of the one-launch op
+// What one launch of the one-launch op adds to a tile's `done` word, all items of the tile together; the word
+// divided by it numbers the launches on the plan (csrc/decode.hip).  More than the shrink items of a tile (16).
+constexpr uint32_t DECODE_TAG_SHIFT = 12;
+constexpr uint32_t DECODE_LAUNCH_WEIGHT = 1u << DECODE_TAG_SHIFT;
+constexpr int ONE_LAUNCH_MAX_POLLS = 4096;   // hard cap on the polls of a bounded wait, whatever the clock says
 
 struct PlanLayout {
   int64_t T, A, max_tiles;
@@ -138,18 +141,15 @@ struct ExpandArgs {
 struct DecodeArgs {
   ShrinkArgs s;               // partial-only shrink: s.partial, s.ksplit >= 2, tile height 16
   ExpandArgs e;               // expand that sums the chunks: e.partial == s.partial, e.ksplit == s.ksplit
-  uint32_t *done;             // [tiles] shrink items finished on this plan so far (only ever counts up)
+  uint32_t *done;             // [tiles] DECODE_LAUNCH_WEIGHT per finished launch on this plan (only ever counts up)
   uint32_t *stamps;           // [tiles][DECODE_MAX_PRODUCERS] (launch tag, XCD) left by each shrink item
   int n_tiles;                // upper bound of the tile count (records past the last tile are zero)
-  int groups_per_chunk;       // groups of 8 tiles whose items the device holds at once
   int n_producers;            // shrink items per tile: ksplit * targets
   int n_consumers;            // expand items per tile: column chunks * targets
-  int resident;               // workgroups the device holds at once: items with a higher id may start late
-  int spin_limit;             // polls of a tile's stamps before an expand item computes the partials itself
+  int spin_limit;             // 10 ns ticks an expand item waits for its tile's stamps before it computes the partials itself
 };
 int launch_decode(hipStream_t st, const DecodeArgs &a, int max_rank, mlora_dtype dt);
 int decode_bn(int max_rank);   // output columns per expand item of the one-launch op
-int decode_resident_workgroups(int max_rank, mlora_dtype dt);   // workgroups of decode_kernel the current device holds at once
 size_t decode_partial_floats(int64_t n_tiles, int n_targets, int ksplit, int64_t rp);
 int launch_plan(hipStream_t st, int32_t *plan, const PlanLayout &L, const int64_t *ids,
                 const int64_t *a_start, const int64_t *a_len, int n_slots, int bm_s, int bm_e);

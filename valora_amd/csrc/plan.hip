@@ -95,7 +95,6 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
   __shared__ int32_t whist[HIST_WORDS];
   __shared__ Quad wsum[PLAN_WAVES + 1];
   __shared__ int s_wmaxr[PLAN_WAVES];
-  __shared__ int s_err;
 
   __shared__ int32_t s_tab[SMALL ? 4 * PLAN_SMALL_A : 1];
   __shared__ int32_t s_rank[SMALL ? PLAN_SMALL_A : 1];
@@ -136,7 +135,6 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
       s_astart[a] = a == tid ? start0 : a_start[a];
     }
   }
-  if (tid == 0) s_err = 0;
   __syncthreads();
   for (int i = tid; i < n_flag_words; i += THREADS) plan[off_counters + i] = 0;
 
@@ -259,10 +257,12 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
       const int k = i - toff[a];
       const int c = cnt[a];
       const int64_t st = start_of(a);
+      // The index has fewer than 2^31 entries (checked on the host), so a start outside 31 bits lies outside the
+      // index whatever it is: it becomes a position no look-up accepts, and the adapter's rows are skipped like
+      // any other row outside the pool.
       const bool st_bad = st < 0 || st > 0x7fffffff;
-      if (st_bad) atomicOr(&s_err, (int)PERR_START_OVERFLOW);
       const int32_t rec[5] = {a, rank_of(a), gstart[a] + k * bm, min(bm, c - k * bm),
-                              st_bad ? INT32_MIN / 2 : (int32_t)st};   // an index position no look-up accepts
+                              st_bad ? INT32_MIN / 2 : (int32_t)st};
       for (int list = 0; list < (one_list ? 2 : 1); ++list) {
         int32_t *tl = (list ? plan + off_tiles_e : tiles) + (int64_t)i * TILE_WORDS;
 #pragma unroll
@@ -291,7 +291,7 @@ __global__ __launch_bounds__(THREADS) void plan_kernel(
     int maxrank = 0;
     for (int wv = 0; wv < N_WAVES; ++wv) maxrank = max(maxrank, s_wmaxr[wv]);
     plan[H_MAXRANK] = maxrank;
-    plan[H_ERR] = s_err;
+    plan[H_RESERVED] = 0;
     plan[H_BM_S] = bm_s;
     plan[H_BM_E] = bm_e;
     plan[H_NACTIVE] = n_active;

@@ -95,7 +95,7 @@ class LoraPlan:
     def header(self) -> dict:
         h = self.buf[:128].view(torch.int32).cpu().tolist()
         names = ["magic", "T", "n_adapters", "n_tiles_shrink", "n_tiles_expand", "n_groups", "max_rank",
-                 "err", "bm_shrink", "bm_expand", "n_active"]
+                 "reserved", "bm_shrink", "bm_expand", "n_active"]
         return dict(zip(names, h))
 
     def perm(self) -> torch.Tensor:
