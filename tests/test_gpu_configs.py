@@ -9,7 +9,7 @@ import torch
 
 from oracle import lora_oracle as O
 from valora_amd import workloads as W
-from tests._util import (assert_parity, max_rank, oracle_target, run_bgmv, run_multi, run_one_launch, run_plan,
+from tests._util import (MAX_ABS, assert_parity, max_rank, oracle_target, run_bgmv, run_multi, run_one_launch, run_plan,
                          run_prefill, run_sgmm)
 
 pytestmark = pytest.mark.gpu
@@ -135,11 +135,30 @@ def test_full_configs_tolerance_accounting(dev, n, names):
     wd = w.to(dev)
     for name in names:
         what = f"config{n}/{name}/full"
-        ma, rl = assert_parity(run_plan(wd, name).cpu(), oracle_target(w, name), what,
-                               unrounded=oracle_target(w, name, round_y=False))
+        got = run_plan(wd, name).cpu()
+        unrounded = oracle_target(w, name, round_y=False)
+        # The strict form of the stated tolerance, no allowance: against the reference semantics "after fp32
+        # accumulation", i.e. the oracle's accumulator before ITS last rounding.  The 16-bit store of y alone moves a
+        # value by up to half the format's spacing, which is 0.0156 for |y| in [4, 8) in bf16 and 0.031 from 8 on: every
+        # element below that magnitude must be within 2e-2 outright, and on ALL elements what is left of the
+        # difference after the largest possible rounding of the store -- the disagreement of the two accumulations
+        # (summation order, and v rounded to the neighbouring 16-bit value where its own accumulations differ in the
+        # last bit) -- must be a small fraction of the tolerance.
+        u = unrounded.double()
+        diff = (got.double() - u).abs()
+        bits = 10 if w.dtype == torch.float16 else 7
+        half = torch.pow(2.0, torch.floor(torch.log2(u.abs().clamp_min(2.0 ** -14))) - bits) / 2
+        fits = half <= MAX_ABS / 1.25           # the format can express the tolerance at this magnitude
+        strict = float(diff[fits].max())
+        assert strict <= MAX_ABS, f"{what}: |got - unrounded oracle| = {strict:.4e} exceeds {MAX_ABS}"
+        accum = float((diff - half).max())
+        assert accum <= MAX_ABS / 4, f"{what}: the accumulations differ by {accum:.4e}"
+        n_coarse = int((~fits).sum())
+        ma, rl = assert_parity(got, oracle_target(w, name), what, unrounded=unrounded)
         over, total = ALLOWANCE[what]
-        print(f"tolerance accounting {what} {w.dtype}: max_abs={ma:.4e} rel_l2={rl:.3e} over_2e-2={over} of {total}",
-              flush=True)
+        print(f"tolerance accounting {what} {w.dtype}: vs unrounded oracle max_abs={strict:.4e} on the {total - n_coarse} "
+              f"elements whose spacing allows 2e-2 ({n_coarse} are coarser), beyond the store's rounding {accum:.2e} on all; "
+              f"vs rounded oracle max_abs={ma:.4e} rel_l2={rl:.3e} over_2e-2={over} of {total}", flush=True)
         if w.dtype == torch.float16:
             assert over == 0, "fp16 results of these magnitudes have no ulp above 2e-2"
 

@@ -124,3 +124,73 @@ def test_entry_points_under_capture_and_rebuild(dev):
         torch.cuda.synchronize()
         assert_parity(y_graph.cpu(), want(ids_b), "replay after the ids were refilled")
     torch.cuda.current_stream().wait_stream(s)
+
+
+def test_warm_up_then_capture_then_refill(dev):
+    """torch's own recipe for graphs: warm up EAGERLY on the static tensors, capture, then `ids.copy_(new batch)` and
+    replay.  The eager warm-up leaves a plan in the cache under the very key the captured calls use; the capture
+    must not reuse it (the graph would then hold no build of its own and keep applying the warm-up batch's
+    adapters), but record a build that every replay runs on whatever the ids tensor holds by then.  The plan and
+    workspace the graph uses must also outlive the cache's own turnover: more than `cache_max_entries` other
+    batches go through the entry points between replays."""
+    from oracle import lora_oracle as O
+    from tests._util import assert_parity
+    from valora_amd import _plan_cache
+    from valora_amd.kernels import dispatch_bgmv
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(78)
+    T, H, R = 160, 1024, 16
+    pool = W.make_pool([16, 8, 16, 8, 16, 16], H, H, dtype, g, True, std=0.05)
+    pd = pool.to(dev)
+    idx = (pd.a_start, pd.a_len, pd.a_loc)
+    batches = [torch.randint(0, 6, (T,), generator=g) for _ in range(3)]
+    x = torch.randn(T, H, generator=g).to(dtype)
+    y0 = torch.randn(T, H, generator=g).to(dtype)
+    xd, ids_d = x.to(dev), batches[0].to(dev)
+    y = y0.to(dev)
+    delta = torch.zeros(T, R, dtype=dtype, device=dev)
+
+    def want(ids):
+        return O.lora_op(y0, x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, 1,
+                         pool.a_scaling)
+
+    def pair():
+        dispatch_bgmv(delta, xd, pd.key_buffer, *idx, ids_d, 1, pd.a_scaling)
+        dispatch_bgmv(y, delta, pd.value_buffer, *idx, ids_d, 1, pd.a_scaling)
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(3):                     # eager warm-up on the static tensors: leaves an eager plan in the cache
+            y.copy_(y0)
+            pair()
+        torch.cuda.synchronize()
+        assert_parity(y.cpu(), want(batches[0]), "eager warm-up")
+        graph = torch.cuda.CUDAGraph()
+        m0 = _plan_cache.misses
+        with torch.cuda.graph(graph, stream=s):
+            pair()
+        assert _plan_cache.misses - m0 == 1, "the capture must record a plan build of its own"
+        for rep, ids in enumerate((batches[1], batches[2], batches[0])):
+            ids_d.copy_(ids.to(dev))
+            y.copy_(y0)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert_parity(y.cpu(), want(ids), f"replay {rep} after the ids were refilled")
+        # turn the cache over with other batches (each a new ids tensor: a new key), then replay again
+        others = []
+        for k in range(_plan_cache.max_entries() + 3):
+            ids_k = torch.randint(0, 6, (T,), generator=g).to(dev)
+            yk, dk = y0.to(dev), torch.zeros(T, R, dtype=dtype, device=dev)
+            dispatch_bgmv(dk, xd, pd.key_buffer, *idx, ids_k, 1, pd.a_scaling)
+            dispatch_bgmv(yk, dk, pd.value_buffer, *idx, ids_k, 1, pd.a_scaling)
+            others.append((ids_k, yk, dk))
+        junk = [torch.randn(1 << 18, device=dev) for _ in range(8)]      # eager allocations that could land on freed memory
+        torch.cuda.synchronize()
+        ids_d.copy_(batches[1].to(dev))
+        y.copy_(y0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert_parity(y.cpu(), want(batches[1]), "replay after the cache turned over")
+        assert all(torch.isfinite(j).all() for j in junk)
+    torch.cuda.current_stream().wait_stream(s)

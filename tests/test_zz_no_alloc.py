@@ -1,9 +1,12 @@
 """GPU: the entry point that allocates nothing (``mlora_dispatch_bgmv_static``) against
-``mlora_dispatch_bgmv`` with a caller-owned workspace: same bits, two calls in a row on the shared built-in
-workspace (the second with a smaller batch), and the size limit."""
+``mlora_dispatch_bgmv`` with a caller-owned workspace and against the oracle: same bits as the former, the
+latter's tolerance, two calls in a row on the shared built-in workspace (the second with a smaller batch), and
+the size limit."""
 import pytest
 import torch
 
+from oracle import lora_oracle as O
+from tests._util import assert_parity
 from valora_amd import _lib, workloads as W
 
 pytestmark = pytest.mark.gpu
@@ -52,6 +55,13 @@ def test_static_workspace_entry_point_matches_dispatch_bgmv(dev, dtype):
         assert torch.equal(d_s, d_w), f"T={T}: shrink differs"
         assert torch.equal(y_s, y_w), f"T={T}: expand differs"
         assert not torch.equal(y_s, y0.cpu()) and bool((d_s != 0.5).any()), "the calls did something"
+        # and the numbers are the operator's (valora/csrc/bgmv/bgmv_impl.cuh:14-207), not merely the sibling's
+        pc, idc = pool.to("cpu"), ids.cpu()
+        want_d = O.bgmv_shrink(torch.full((T, narrow), 0.5, dtype=dtype), x.cpu(), pc.key_buffer, pc.a_start, pc.a_len,
+                               pc.a_loc, idc, 2)
+        want_y = O.bgmv_expand(y0.cpu(), v.cpu(), pc.value_buffer, pc.a_start, pc.a_len, pc.a_loc, idc, 2, pc.a_scaling)
+        assert_parity(d_s, want_d, f"static workspace, T={T}: shrink vs oracle")
+        assert_parity(y_s, want_y, f"static workspace, T={T}: expand vs oracle")
 
 
 def test_static_workspace_size_limit(dev):

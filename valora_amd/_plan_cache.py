@@ -16,8 +16,10 @@ an equal key really means the same memory, and ``_version`` says it has not been
 PyTorch since.  Tensors created under ``torch.inference_mode`` carry no version counter; they are
 cached by address alone while ``cache_inference_tensors()`` is true (an in-place write to such a
 tensor is then not noticed).  Writes that bypass PyTorch's bookkeeping (a foreign kernel given the
-raw pointer) are never seen: ``set_enabled(False)`` turns the reuse off.  A plan whose build was only
-recorded into a stream capture serves that capture alone.
+raw pointer) are never seen: ``set_enabled(False)`` turns the reuse off.  A plan serves the context it was
+built in and no other: one whose build was only recorded into a stream capture serves that capture alone, and
+one cut eagerly (a warm-up before the capture) is not used under capture -- the graph records a build of its own,
+so a replay cuts the tiles of whatever the ids tensor holds by then, in buffers that live as long as the graph.
 
 At most ``max_entries()`` plans are kept (least recently used first out); each holds its workspace
 (``mlora_workspace_bytes``: KBs at decode sizes, tens of MB for long prefills) and the small index

@@ -102,8 +102,7 @@ void key_scalar(Key &k, int64_t v) {
   k.s[k.ns++] = v;
 }
 
-// Id of the capture `stream` is recording into, 0 if it is not capturing.  A plan whose build was only
-// recorded (not run) is valid for launches recorded into the same capture, and for nothing else.
+// Id of the capture `stream` is recording into, 0 if it is not capturing.
 unsigned long long capture_id(hipStream_t stream) {
   hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
   unsigned long long id = 0;
@@ -114,13 +113,21 @@ unsigned long long capture_id(hipStream_t stream) {
   return st == hipStreamCaptureStatusActive ? (id ? id : ~0ull) : 0;
 }
 
+// The entry for `key` that may serve a call on `stream`.  A plan is valid in the context it was built in and in no
+// other: one cut eagerly (capture == 0) for eager calls only -- recorded into a capture it would leave the graph
+// without a build of its own, and every replay would reuse the tiles of the batch that happened to be in the ids
+// tensor at warm-up, whatever the caller has written there since, from buffers this cache is free to drop -- and one
+// whose build was only recorded (capture != 0) for calls recorded into the same capture.  A call under capture
+// that finds none of its own builds a fresh plan inside the capture (its buffers come from the graph's memory pool
+// and live as long as the graph); entries of a capture that is over are dropped when their key comes up again.
 Entry *find(const Key &key, hipStream_t stream, bool native) {
+  const unsigned long long now = native ? capture_id(stream) : 0;
   for (size_t i = g_entries.size(); i-- > 0;) {
     Entry *e = g_entries[i].get();
     if (!(e->key == key)) continue;
-    if (native && e->capture != 0 && e->capture != capture_id(stream)) {
-      g_entries.erase(g_entries.begin() + i);  // built inside another capture: its tiles may never have been cut
-      return nullptr;
+    if (native && e->capture != now) {
+      if (e->capture != 0) g_entries.erase(g_entries.begin() + i);  // recorded into another capture: never cut eagerly
+      continue;
     }
     if (i + 1 != g_entries.size()) {
       std::unique_ptr<Entry> keep = std::move(g_entries[i]);
