@@ -51,7 +51,8 @@ def parse():
                     help="first run one plain device copy of this many MiB: a kernel of known traffic to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings with")
     ap.add_argument("--only-config", type=int, default=0,
-                    help="with --all-configs: report this benchmark configuration only (1, 3, 4 or 5)")
+                    help="with --all-configs: report this benchmark configuration only (1, 3, 4, 5, or 2: the headline's "
+                         "decode batch on all seven projections of a layer)")
     ap.add_argument("--only-target", default=None,
                     help="with --all-configs --only-config N: time this target only (q, k, v, o, gate, up, down) and "
                          "no multi-target group, so that a profile of the run holds one shape per kernel")
@@ -152,13 +153,14 @@ COLD_BYTES = 1 << 30   # four times the 256 MB last-level cache of the MI355X
 
 
 def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0, only_target=None):
-    """Per-target timing of the other benchmark configurations (report only; the JSON line of the
-    default run is config 2).  Each target's shrink+expand is replayed back to back on 4 copies of y
+    """Per-target timing of the other benchmark configurations and of the headline's decode batch on all seven
+    projections of a layer (report only; the JSON line of the default run is config 2's q).  Each target's shrink+expand is replayed back to back on 4 copies of y
     so that the read-modify-write does not hit the same lines (`us`: x and the pool may sit in the
     last-level cache), and once more over 1 GiB of x / y copies (`us_cold`)."""
     report = {}
-    for n in ((only,) if only else (1, 3, 4, 5)):
-        w = W.CONFIGS[n]()
+    for n in ((only,) if only else (1, 2, 3, 4, 5)):
+        # 2: the headline's decode batch with LoRA on all seven projections of a layer (the headline itself is its q)
+        w = W.decode_layer() if n == 2 else W.CONFIGS[n]()
         wd = w.to(dev)
         R = max(w.targets[0].pool.ranks)
         rows = {}

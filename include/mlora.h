@@ -52,8 +52,10 @@ enum {
                                  mlora_one_launch_scratch_bytes(), 128-byte aligned (the partials are
                                  handed over in cache lines that belong to one tile each; a scratch
                                  buffer aligned to less, an empty index or an empty pool make the call
-                                 run as two launches).  Any batch size: items the device cannot hold
-                                 from the start take part in the hand-off like the others.
+                                 run as two launches, and so does a call with more than 16 expand items
+                                 per tile -- 512-column chunks (256 above rank 32) x targets -- where two
+                                 launches measured faster).  Any batch size: items the device cannot
+                                 hold from the start take part in the hand-off like the others.
                                  Bit-identical to the two-launch op with MLORA_REDUCE_IN_EXPAND and the
                                  same ksplit.  Launches that share a plan must not overlap in time.  */
   MLORA_ONE_LAUNCH_NO_WAIT = 4, /* with MLORA_ONE_LAUNCH: expand items do not wait at all and always

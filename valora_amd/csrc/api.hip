@@ -34,6 +34,8 @@ int decode_bn(int max_rank);   // output columns per expand item of the one-laun
 // items that wait for them and run for a few microseconds, so a healthy launch never gets near the bound; it only
 // limits how long a workgroup holds its slot when the producers are held up (a device shared with other work).
 constexpr int ONE_LAUNCH_WAIT_TICKS = 3000;
+// expand items per tile up to which a call that asks for one launch gets it (see mlora_lora_apply_multi)
+constexpr int ONE_LAUNCH_MAX_EXPAND_ITEMS = 16;
 
 namespace {
 
@@ -427,6 +429,14 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
   // same ksplit, which gives the same bits.
   bool use_decode = one_launch && aligned128(scratch) && pool_a->a_loc_len > 0 && pool_a->w_rows > 0;
   for (int i = 0; use_decode && i < n_targets; ++i) use_decode = targets[i].w_b_rows > 0;
+  // Where the one-launch op pays is a matter of the expand items per tile (column chunks x targets), measured on 256
+  // decode tokens over 64 adapters: up to 16 of them (one or two 4096-wide targets, an 11008 -> 4096 one) it is
+  // 2 - 2.5 us faster than two launches, with more (q+k+v: 24, one 4096 -> 11008 target: 22) the expand half is the
+  // longer one and the column-looping expand launch does it 3 us faster than these items do.
+  if (use_decode) {
+    const int64_t bn = decode_bn((int)max_rank);
+    use_decode = (h_out + bn - 1) / bn * n_targets <= ONE_LAUNCH_MAX_EXPAND_ITEMS;
+  }
   if (ksplit < 1 || ksplit > 64) return fail(MLORA_ERR_INVALID, "lora_apply_multi: ksplit=%d outside [1,64]", ksplit);
   const size_t per_target = scratch_bytes(T, max_rank, ksplit);
   const size_t scratch_need = use_decode ? mlora_one_launch_scratch_bytes(T, plan->n_adapters, max_rank, ksplit, n_targets)

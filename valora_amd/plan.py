@@ -48,7 +48,6 @@ class LoraPlan:
         rie = cfg.reduce_in_expand if reduce_in_expand is None else reduce_in_expand
         self.flags = _lib.REDUCE_IN_EXPAND if rie else 0
         self.one_launch = bool(cfg.one_launch if one_launch is None else one_launch)
-        self._one_launch_by_table = one_launch is None
         if self.one_launch and (self.max_rank > 64 or bm_shrink not in (None, 16) or bm_expand not in (None, 16)):
             if one_launch:
                 raise RuntimeError("No suitable kernel. the one-launch op needs 16-token tiles and max_rank <= 64")
@@ -178,15 +177,9 @@ class LoraPlan:
         tg = (_lib.Target * n)()
         for i in range(n):
             tg[i] = _lib.Target(_lib.ptr(ys[i]), _lib.ptr(vbs[i]), vbs[i].numel() // h_out, int(slots[i]))
+        # (a call whose expand half is more than 16 items per tile -- q+k+v, a 4096 -> 11008 target -- is run as two
+        # launches by the library whatever the flag says: same tiles, same split, same bits)
         flags = self.flags
-        if self.one_launch and self._one_launch_by_table and n > 1:
-            # the table's mark was measured on one target.  With several, the one-launch op still pays up to 16
-            # expand items per tile (two 4096-wide targets: 6.5-7.9 us against 7.5-9.2 as two launches, 1-64 tokens);
-            # beyond that two launches win (three rank-64 targets of 8 tokens: 15.0 against 18.3 us, gate+up 4096 ->
-            # 11008: 7.9 against 8.9).  Same tiles, same split, same bits either way.
-            chunk = 512 if self.max_rank <= 32 else 256
-            if n * ((h_out + chunk - 1) // chunk) > 16:
-                flags &= ~(_lib.ONE_LAUNCH | _lib.ONE_LAUNCH_NO_WAIT)
         _lib.check(_lib.lib().mlora_lora_apply_multi(
             _lib.current_stream(self.device), self.handle, _lib.ptr(self.scratch), self.scratch.numel(), _lib.ptr(x),
             self.T, h_in, h_out, self.max_rank, pa, n, tg, _lib.ptr(scales), int(self.ksplit), flags,

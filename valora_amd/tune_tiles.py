@@ -47,7 +47,13 @@ def _time(fn, reps=30, warm=3) -> float:
     return e0.elapsed_time(e1) * 1e3 / reps
 
 
-def synthetic_batch(n_tokens: int, n_adapters: int, rank: int, hidden: int, dtype, seed: int):
+def down_projection_width(hidden: int) -> int:
+    """Output width of the target whose INPUT is `hidden` wide when that is an MLP width (a down projection back to
+    the model width: 11008 / 13824 / 14336 -> 4096 or 5120-ish, 28672 -> 8192); a model width maps to itself."""
+    return hidden if hidden <= 8192 else 4096 if hidden < 20000 else 8192
+
+
+def synthetic_batch(n_tokens: int, n_adapters: int, rank: int, hidden: int, dtype, seed: int, h_out: int = 0):
     """Decode-like (one token per request) up to 1024 tokens; above, requests of 128 tokens, or shorter ones where
     that many would be fewer than the adapter bucket stands for (2048 tokens over 128 adapters: 16-token requests,
     the decode-heavy mix of a continuous batch); adapters drawn Zipf(0.7) per request."""
@@ -56,7 +62,7 @@ def synthetic_batch(n_tokens: int, n_adapters: int, rank: int, hidden: int, dtyp
     n_req = max(1, n_tokens // req_len)
     req_ids = W.zipf_ids(n_adapters, n_req, 0.7, g)
     ids = torch.repeat_interleave(req_ids, req_len)
-    pool = W.make_pool([rank] * n_adapters, hidden, hidden, dtype, g, paged=True)
+    pool = W.make_pool([rank] * n_adapters, hidden, h_out or hidden, dtype, g, paged=True)
     x = torch.randn(ids.numel(), hidden, generator=g).to(dtype)
     return ids, pool, x
 
@@ -159,11 +165,13 @@ def tune_tall_shrink(dev, n_tokens, n_adapters, rank, hidden, entry, dtype=torch
 
 def tune_one_launch(dev, n_tokens, n_adapters, rank, hidden, entry, dtype=torch.float16, copies=4):
     """Does the one-launch op (shrink and expand items of one grid, 16-token tiles) beat the two-launch entry of
-    this shape?  Returns the entry to keep and both timings.  Only decode-like shapes qualify: rank <= 64 and a
-    grid the device holds at once (the library runs larger ones as two launches anyway)."""
-    ids, pool, x = synthetic_batch(n_tokens, n_adapters, rank, hidden, dtype, seed=n_tokens + n_adapters + rank)
+    this shape?  Returns the entry to keep and both timings.  Only decode-like shapes qualify: rank <= 64.  The
+    library runs a call with more than 16 expand items per tile as two launches whatever the entry says, so an
+    MLP-wide `hidden` is measured as what it is the input of, a down projection (to a 4096- or 8192-wide output)."""
+    h_out = down_projection_width(hidden)
+    ids, pool, x = synthetic_batch(n_tokens, n_adapters, rank, hidden, dtype, seed=n_tokens + n_adapters + rank, h_out=h_out)
     ids, x, p = ids.to(dev), x.to(dev), pool.to(dev)
-    ys = [torch.zeros(ids.numel(), hidden, dtype=dtype, device=dev) for _ in range(copies)]
+    ys = [torch.zeros(ids.numel(), h_out, dtype=dtype, device=dev) for _ in range(copies)]
     idx = (p.a_start, p.a_len, p.a_loc)
 
     def op_us(**kw):
@@ -196,7 +204,7 @@ def main():
     ap.add_argument("--ranks", type=int, nargs="+", default=list(tt.RANK_BUCKETS))
     ap.add_argument("--out", default=tt.TABLE_PATH)
     ap.add_argument("--one-launch", action="store_true",
-                    help="revisit the existing entries of decode-like shapes (<= 1024 tokens, rank <= 64; the protected "
+                    help="revisit the existing entries of decode-like shapes (<= 2048 tokens, rank <= 64; the protected "
                          "ones too) and mark those where the one-launch op is faster than the entry's two launches")
     ap.add_argument("--tall-shrink", action="store_true",
                     help="revisit the existing entries above 4096 tokens that use 128-token shrink tiles (rank <= 64, summed "
@@ -236,7 +244,7 @@ def main():
                     json.dump(table, f, indent=1)
             continue
         if args.one_launch:
-            if k in entries and n_tokens <= 1024 and rank <= 64:
+            if k in entries and n_tokens <= 2048 and rank <= 64:
                 new, two, one = tune_one_launch(dev, n_tokens, min(n_adapters, max(1, n_tokens)), rank, hidden, entries[k])
                 # a protected entry was tuned on its real workload: the synthetic batch (which may not fit the
                 # device as one grid where the real one does) can add the mark there, never take it away
