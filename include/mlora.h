@@ -66,11 +66,16 @@ enum {
                                  the others' partials out of the L2 it shares with them, or -- when they
                                  did not all run on its XCD -- computes them itself.  This flag makes
                                  every tile take the second path (made testable; same results, slower) */
-  MLORA_EXPAND_COLUMN_LOOP = 16 /* expand of a plan with 16-token expand tiles: a workgroup walks over two
+  MLORA_EXPAND_COLUMN_LOOP = 16, /* expand of a plan with 16-token expand tiles: a workgroup walks over two
                                  256-column chunks of its tile instead of owning one.  The library does
                                  this by itself where the grid would otherwise be several times what the
                                  device holds (decode batches with many targets or wide outputs); the flag
                                  forces it for any size (made testable; same results)                    */
+  MLORA_ONE_LAUNCH_NEVER_READY = 32  /* with MLORA_ONE_LAUNCH: expand items look for a stamp that no shrink item
+                                 leaves, so every one of them waits out its bound (30 us) and then computes
+                                 its tile's partials itself: the way out of the bounded wait made testable
+                                 and measurable from the host; every kernel still ends normally, same
+                                 results, slower                                                          */
 };
 
 /* What the kernels can vary per batch shape (see mlora_tile_lookup). */

@@ -327,3 +327,79 @@ def test_two_streams_with_a_plan_each_run_side_by_side(dev):
         for k, (side, out) in enumerate(zip(sides, outs)):
             for l in range(L):
                 assert torch.equal(out[l], side[4][l]), f"repetition {rep}, stream {k}, layer {l}"
+
+
+def test_a_wait_that_runs_out(dev):
+    """Every expand item looks for a stamp nobody leaves (a flag from the host), waits out its bound and then computes
+    its tile's partials itself: the whole way out of the bounded wait, on a healthy device, with every kernel ending
+    normally.  Same bits as two launches; the op takes the bound (30 us) plus the recomputation, not more."""
+    w = W.config2(hidden=1024, n_tokens=64, n_adapters=16)
+    wd = w.to(dev)
+    t = wd.target("q"); p = t.pool
+    R = max(p.ranks)
+    slow = LoraPlan(wd.ids, p.a_start, p.a_len, R, hidden=1024, one_launch=True, ksplit=4, one_launch_never_ready=True)
+    one, two = _pair(wd, "q", R, 1024, 4)
+    outs = []
+    for plan in (slow, one, two):
+        y = wd.y0["q"].clone()
+        plan.apply(y, wd.x[1024], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
+        outs.append(y)
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[2]) and torch.equal(outs[1], outs[2])
+
+    def timed(plan, reps=20):
+        y = wd.y0["q"].clone()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            plan.apply(y, wd.x[1024], p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+
+    us_slow, us_fast = timed(slow), timed(one)
+    print(f"one-launch op: {us_fast:.1f} us; with every wait running out: {us_slow:.1f} us", flush=True)
+    assert us_slow > 30.0, "the waits must really have run to their bound"
+    assert us_slow < 150.0, "and not past it: 30 us of waiting, then the tile's partials computed in place"
+
+
+def test_operands_the_one_launch_kernel_cannot_take_run_as_two_launches(dev):
+    """The one-launch kernel reads element 0 of the index and of every target's pool where it has nothing to fetch,
+    and hands partials over in cache lines of the scratch buffer: an empty index, a target pool of zero rows or a
+    scratch buffer that is only 16-byte aligned make the library run the call as two launches (whose loads are
+    guarded).  No fault, the documented result: rows whose weights cannot be found keep their values."""
+    from valora_amd import _lib
+    L = _lib.lib()
+    w = W.config2(hidden=512, n_tokens=48, n_adapters=12)
+    wd = w.to(dev)
+    t = wd.target("q"); p = t.pool
+    R = max(p.ranks)
+    plan = LoraPlan(wd.ids, p.a_start, p.a_len, R, hidden=512, one_launch=True, ksplit=4)
+    code = _lib.dtype_code(w.dtype)
+    st = _lib.current_stream(dev)
+    x, y0 = wd.x[512], wd.y0["q"]
+    want = y0.clone()
+    plan.apply(want, x, p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
+
+    def call(pa, tg, scratch_ptr, scratch_bytes):
+        y = y0.clone()
+        tgs = (_lib.Target * 1)(_lib.Target(_lib.ptr(y), tg[0], tg[1], t.slot))
+        _lib.check(L.mlora_lora_apply_multi(st, plan.handle, scratch_ptr, scratch_bytes, _lib.ptr(x), w.T, 512, 512, R, pa, 1,
+                                            tgs, _lib.ptr(p.a_scaling), plan.ksplit, plan.flags, code))
+        torch.cuda.synchronize()
+        return y
+
+    pa = _lib.make_pool(p.key_buffer, p.a_start, p.a_len, p.a_loc, 512, 4)
+    full = (_lib.ptr(p.value_buffer), p.value_buffer.numel() // 512)
+    sp, sb = _lib.ptr(plan.scratch), plan.scratch.numel()
+    assert torch.equal(call(pa, full, sp, sb), want)
+    # scratch that starts 16 bytes into a line
+    off = _lib.c_void_p(plan.scratch.data_ptr() + 16)
+    assert torch.equal(call(pa, full, off, sb - 16), want), "a 16-byte aligned scratch buffer gives the same bits"
+    # a B pool of zero rows: nothing can be found, y keeps its values
+    assert torch.equal(call(pa, (_lib.ptr(p.value_buffer), 0), sp, sb), y0)
+    # an empty index: no adapter has rows
+    empty = torch.empty(0, dtype=torch.long, device=dev)
+    pe = _lib.make_pool(p.key_buffer, p.a_start, p.a_len, empty, 512, 4)
+    assert torch.equal(call(pe, full, sp, sb), y0)

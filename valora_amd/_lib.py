@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libmlora.so")
 
 MLORA_F16, MLORA_BF16 = 0, 1
 SHRINK_OVERWRITE, SHRINK_ZERO_PAD, SHRINK_ACCUMULATE = 0, 1, 2
-REDUCE_IN_EXPAND, ONE_LAUNCH, ONE_LAUNCH_NO_WAIT, SHRINK_RECOMPUTE, EXPAND_COLUMN_LOOP = 1, 2, 4, 8, 16
+REDUCE_IN_EXPAND, ONE_LAUNCH, ONE_LAUNCH_NO_WAIT, SHRINK_RECOMPUTE, EXPAND_COLUMN_LOOP, ONE_LAUNCH_NEVER_READY = 1, 2, 4, 8, 16, 32
 
 # every symbol include/mlora.h declares
 SYMBOLS = [

@@ -523,6 +523,7 @@ int mlora_lora_apply_multi(void *stream, const mlora_plan *plan, void *scratch, 
     d.n_producers = ksplit * n_targets;
     d.n_consumers = d.e.n_ochunks * n_targets;
     d.spin_limit = (flags & MLORA_ONE_LAUNCH_NO_WAIT) ? 0 : ONE_LAUNCH_WAIT_TICKS;
+    d.never_ready = (flags & MLORA_ONE_LAUNCH_NEVER_READY) ? 1 : 0;
     return launch_decode((hipStream_t)stream, d, (int)max_rank, dtype);
   }
   return launch_expand((hipStream_t)stream, e, (int)max_rank, tiles_upper(T, plan->n_adapters, plan->bm_expand),

@@ -219,7 +219,8 @@ __global__ __launch_bounds__(256, 3) void decode_kernel(const int32_t *tiles_bas
   // fields early as well measured 0.04 us slower, the target's operands on top of that another 0.08 us)
   if (cnt <= 0) return;   // records past the last tile are zero
   const int32_t *__restrict__ perm = plan_words + off_perm;
-  const uint32_t want_stamp = stamp_of(done0, xcd_id());
+  // (never_ready: a stamp with the top bit set, which no shrink item leaves -- the wait runs to its bound)
+  const uint32_t want_stamp = stamp_of(done0, xcd_id()) | (a.never_ready ? 0x80000000u : 0u);
   uint32_t *const stamps = stamps_base + (int64_t)tile_idx * DECODE_MAX_PRODUCERS;
   float *const tile_partial = partial_base + (int64_t)tile_idx * n_producers * 16 * rp;
   const int z = item / n_ochunks, oc = item - z * n_ochunks;

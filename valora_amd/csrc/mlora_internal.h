@@ -146,6 +146,7 @@ struct DecodeArgs {
   int n_tiles;                // upper bound of the tile count (records past the last tile are zero)
   int n_producers;            // shrink items per tile: ksplit * targets
   int n_consumers;            // expand items per tile: column chunks * targets
+  int never_ready;            // tests: expand items look for a stamp nobody leaves and wait out their bound
   int spin_limit;             // 10 ns ticks an expand item waits for its tile's stamps before it computes the partials itself
 };
 int launch_decode(hipStream_t st, const DecodeArgs &a, int max_rank, mlora_dtype dt);

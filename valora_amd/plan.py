@@ -23,13 +23,15 @@ class LoraPlan:
                  n_slots: int = 4, hidden: int = 4096, bm_shrink: Optional[int] = None,
                  bm_expand: Optional[int] = None, ksplit: Optional[int] = None,
                  reduce_in_expand: Optional[bool] = None, one_launch: Optional[bool] = None,
-                 one_launch_no_wait: bool = False, shrink_recompute: bool = False, expand_column_loop: bool = False):
+                 one_launch_no_wait: bool = False, shrink_recompute: bool = False, expand_column_loop: bool = False,
+                 one_launch_never_ready: bool = False):
         """``ids``: int64 per-token adapter index (negative = no adapter); ``a_start`` / ``a_len``:
         the pool index (``a_len = n_slots * rank``); ``max_rank``: widest rank among the resident
         adapters (the reference's ``max_lora_dim``, lora_unordered_batch_infer.py:181-182).
         ``one_launch``: shrink and expand as work items of one grid (decode-like batches; forces
         16-token tiles, needs ``max_rank <= 64``); ``None`` takes the tile table's choice.
-        ``one_launch_no_wait`` makes every expand item take its give-up path, ``shrink_recompute`` makes the
+        ``one_launch_no_wait`` makes every expand item take its give-up path at once, ``one_launch_never_ready`` after
+        waiting out its bound, ``shrink_recompute`` makes the
         128-token shrink sum its K chunks by computing them all in one workgroup, ``expand_column_loop`` makes the
         expand of 16-token tiles walk over two column chunks per workgroup whatever the grid size (all for tests)."""
         if not ids.is_cuda:
@@ -55,7 +57,8 @@ class LoraPlan:
         if self.one_launch:
             self.bm_shrink = self.bm_expand = 16
             self.ksplit = max(2, self.ksplit)
-            self.flags = _lib.REDUCE_IN_EXPAND | _lib.ONE_LAUNCH | (_lib.ONE_LAUNCH_NO_WAIT if one_launch_no_wait else 0)
+            self.flags = (_lib.REDUCE_IN_EXPAND | _lib.ONE_LAUNCH | (_lib.ONE_LAUNCH_NO_WAIT if one_launch_no_wait else 0) |
+                          (_lib.ONE_LAUNCH_NEVER_READY if one_launch_never_ready else 0))
         if shrink_recompute:
             self.flags |= _lib.SHRINK_RECOMPUTE
         if expand_column_loop:
