@@ -59,14 +59,12 @@ __device__ __forceinline__ void store_v(const ShrinkArgs &p, int pos, int t, int
 template <typename T>
 __device__ __forceinline__ void shrink_epilogue(const ShrinkArgs &p, const float *tile, int ld, int s, int pos0,
                                                 int cnt, int r, const int32_t *perm) {
-  // `tile` has ld columns per row (the rank blocks the tile was computed with, at least the tile's rank);
-  // columns from there to rp are zero
   const int tid = threadIdx.x;
   if (p.ksplit == 1) {
     const int n_el = cnt * p.rp;
     for (int e = tid; e < n_el; e += 256) {
       const int row = e / p.rp, col = e - row * p.rp;
-      store_v<T>(p, pos0 + row, p.out_by_token ? perm[pos0 + row] : 0, r, col, col < ld ? tile[row * ld + col] : 0.f);
+      store_v<T>(p, pos0 + row, p.out_by_token ? perm[pos0 + row] : 0, r, col, tile[row * ld + col]);
     }
     return;
   }
@@ -76,7 +74,7 @@ __device__ __forceinline__ void shrink_epilogue(const ShrinkArgs &p, const float
   for (int e = tid; e < n_vec; e += 256) {
     const int row = e / quarter, c4 = e - row * quarter;
     const float *src = tile + row * ld + 4 * c4;
-    part[e] = 4 * c4 < ld ? f32x4{src[0], src[1], src[2], src[3]} : f32x4{0.f, 0.f, 0.f, 0.f};
+    part[e] = f32x4{src[0], src[1], src[2], src[3]};
   }
 }
 
@@ -144,34 +142,9 @@ __global__ __launch_bounds__(256) void shrink_kernel(const int32_t *tiles_base, 
   const int32_t *__restrict__ perm = p.plan + p.off_perm;
   const int kbeg = s * p.kchunk;
   const int kend = min(p.h_in, kbeg + p.kchunk);
-  // The kernel is instantiated for the widest rank of the batch (NB blocks of 16), which also fixes how many K steps
-  // a wave keeps in flight (the registers are shared between operand loads and accumulators).  A tile of a narrower
-  // adapter runs the instantiation for ITS rank with as many K steps in flight as the wide one's loads leave room
-  // for: fewer accumulators, more of K requested at once, the same order of accumulation (same bits).  The result
-  // tile then has ldt = 16 * (its rank blocks) columns per row and sits where that instantiation's second buffer is.
-  constexpr int LOADS = shrink_steps_in_flight(MB, NB) * (MB + NB);   // 16-byte loads per lane the kernel is built for
-  int ldt = NB * 16;
-  const float *otile = red[1];
-  if (NB >= 2 && r <= 16 && LOADS / (MB + 1) > shrink_steps_in_flight(MB, NB)) {
-    auto redn = reinterpret_cast<float(*)[MB * 1 * 256]>(&red[0][0]);
-    shrink_tile_to_lds<T, MB, 1, LOADS / (MB + 1)>(p.x, p.h_in, p.pool, p.slot, perm, r, pos0, cnt, astart, kbeg, kend, redn);
-    ldt = 16;
-    otile = redn[1];
-  } else if (NB >= 4 && r <= 32 && LOADS / (MB + 2) > shrink_steps_in_flight(MB, NB)) {
-    auto redn = reinterpret_cast<float(*)[MB * 2 * 256]>(&red[0][0]);
-    shrink_tile_to_lds<T, MB, 2, LOADS / (MB + 2)>(p.x, p.h_in, p.pool, p.slot, perm, r, pos0, cnt, astart, kbeg, kend, redn);
-    ldt = 32;
-    otile = redn[1];
-  } else if (NB >= 8 && r <= 64 && LOADS / (MB + 4) > shrink_steps_in_flight(MB, NB)) {
-    auto redn = reinterpret_cast<float(*)[MB * 4 * 256]>(&red[0][0]);
-    shrink_tile_to_lds<T, MB, 4, LOADS / (MB + 4)>(p.x, p.h_in, p.pool, p.slot, perm, r, pos0, cnt, astart, kbeg, kend, redn);
-    ldt = 64;
-    otile = redn[1];
-  } else {
-    shrink_tile_to_lds<T, MB, NB>(p.x, p.h_in, p.pool, p.slot, perm, r, pos0, cnt, astart, kbeg, kend, red);
-  }
+  shrink_tile_to_lds<T, MB, NB>(p.x, p.h_in, p.pool, p.slot, perm, r, pos0, cnt, astart, kbeg, kend, red);
   if (!p.reduce_here || p.ksplit == 1) {
-    shrink_epilogue<T>(p, otile, ldt, s, pos0, cnt, r, perm);
+    shrink_epilogue<T>(p, red[1], NB * 16, s, pos0, cnt, r, perm);
     return;
   }
 
@@ -189,15 +162,12 @@ __global__ __launch_bounds__(256) void shrink_kernel(const int32_t *tiles_base, 
   // (Worth it for small tiles only: one workgroup reads ksplit x tile x prp x 4 bytes at L2 latency.  For
   // 128-token tiles of rank 64 that is 256 KB and measured 8.5 us, against 3.7 us for the reduce launch.)
   const int tid = threadIdx.x;
-  const int pq = p.prp >> 2;
-  // only the columns of the tile's own rank travel (r is a multiple of 8): a rank-16 tile of a rank-64 batch leaves
-  // and reads a quarter of the bytes; what v holds beyond them is zero
-  const int quarter = (r + 3) >> 2 < (p.rp >> 2) ? (r + 3) >> 2 : (p.rp >> 2);
+  const int quarter = p.rp >> 2, pq = p.prp >> 2;
   {
     f32x4 *part = reinterpret_cast<f32x4 *>(p.partial + ((int64_t)s * p.T + pos0) * p.prp);
     for (int e = tid; e < cnt * quarter; e += 256) {
       const int row = e / quarter, c4 = e - row * quarter;
-      const float *src = otile + row * ldt + 4 * c4;
+      const float *src = red[1] + row * (NB * 16) + 4 * c4;
       part[row * pq + c4] = f32x4{src[0], src[1], src[2], src[3]};
     }
   }
@@ -223,11 +193,10 @@ __global__ __launch_bounds__(256) void shrink_kernel(const int32_t *tiles_base, 
     // v[row, :] = T(0 + p_0 + p_1 + ...): the order shrink_reduce_kernel uses
     const f32x4 *src = reinterpret_cast<const f32x4 *>(p.partial + (int64_t)pos0 * p.prp);
     const int64_t sstride = (int64_t)p.T * pq;
-    const int all_q = p.rp >> 2;
-    for (int e = tid; e < cnt * all_q; e += 256) {
-      const int row = e / all_q, c4 = e - row * all_q;
+    for (int e = tid; e < cnt * quarter; e += 256) {
+      const int row = e / quarter, c4 = e - row * quarter;
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
-      for (int s0 = 0; c4 < quarter && s0 < p.ksplit; s0 += 8) {
+      for (int s0 = 0; s0 < p.ksplit; s0 += 8) {
         f32x4 q[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u)

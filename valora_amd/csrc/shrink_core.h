@@ -20,14 +20,7 @@ namespace mlora {
 // Leaves the fp32 result of K range [kbeg, kend) in red[1], row-major with row stride NB*16
 // (rows = tokens of the tile, columns = rank); every thread of the workgroup must call it, and all
 // have passed a barrier when it returns.
-// K steps a wave keeps in flight for MB token blocks and NB rank blocks: MB + NB 16-byte loads per lane and step
-constexpr int shrink_steps_in_flight(int mb, int nb) {
-  return (mb + nb <= 2) ? 8 : (mb + nb <= 4) ? 4 : (mb + nb <= 8) ? 2 : 1;
-}
-
-// UU: K steps in flight, 0 = the rule above (a caller that runs a narrower instantiation inside a kernel built for
-// a wider one passes what fits the wider one's register budget)
-template <typename T, int MB, int NB, int UU = 0>
+template <typename T, int MB, int NB>
 __device__ __forceinline__ void shrink_tile_to_lds(const uint16_t *__restrict__ x, int h_in, const PoolDev &pool,
                                                    int slot, const int32_t *__restrict__ perm, int r, int pos0,
                                                    int cnt, int astart, int kbeg, int kend,
@@ -71,7 +64,7 @@ __device__ __forceinline__ void shrink_tile_to_lds(const uint16_t *__restrict__ 
   // would still feed its stale registers into the matrix core.  Lanes past the end load zeros.
   // (Whole 128-byte lines per wave and step -- 64 K elements, two loads per lane -- measured the same to
   // slightly slower than these half lines.)
-  constexpr int U = UU > 0 ? UU : shrink_steps_in_flight(MB, NB);
+  constexpr int U = (MB + NB <= 2) ? 8 : (MB + NB <= 4) ? 4 : (MB + NB <= 8) ? 2 : 1;
   for (int kb0 = kbeg + wave * 32; kb0 < kend; kb0 += 128 * U) {
     u32x4 xa[U][MB], wb[U][NB];
 #pragma unroll
