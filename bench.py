@@ -756,7 +756,16 @@ def main():
     sh_ms, _ = time_graph(torch, shrink_only, reps, 5, use_graph)
     ex_ms, _ = time_graph(torch, expand_only, reps, 5, use_graph)
     op_ms, _ = time_graph(torch, layers_only, reps, 5, use_graph)
-    plan_ms, _ = time_graph(torch, plan.rebuild, reps, 5, use_graph)
+    # one plan build: 32 builds back to back in one graph (what the build costs as a node of a step's graph: its
+    # kernel), and a graph that holds nothing but one build (what a replay of a one-kernel graph costs: mostly the
+    # graph launch itself, which varies from box to box and is not the build's)
+
+    def plans_32():
+        for _ in range(32):
+            plan.rebuild()
+
+    plan_ms = time_graph(torch, plans_32, reps, 5, use_graph)[0] / 32
+    plan_alone_ms, _ = time_graph(torch, plan.rebuild, reps, 5, use_graph)
     sh_us, ex_us, op_us = sh_ms * 1e3 / L, ex_ms * 1e3 / L, op_ms * 1e3 / L
 
     s_el = 2
@@ -796,6 +805,8 @@ def main():
         "hbm_frac": round(bytes_op / (us_per_layer * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
         "roofline": roofline,
         "plan_us": round(plan_ms * 1e3, 3),
+        "plan_us_is": "one mlora_build_plan as a node among others of a graph (32 builds back to back in one graph, per build)",
+        "plan_us_one_kernel_graph": round(plan_alone_ms * 1e3, 3),
     }
     if not args.no_extras:
         out["extra"] = bench_extras(torch, W, LoraPlan, dev, L, w, wd, kb, vb, xs, ys, use_graph, reps, args.no_step5)
