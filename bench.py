@@ -27,7 +27,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE),
 # scaled by the same counters' reading for a plain copy of known size; None until measured.
-MEASURED_TRAFFIC_BYTES = {"decode_kernel": 23_580_000, "expand_kernel": 13_050_000,
+MEASURED_TRAFFIC_BYTES = {"decode_kernel": 23_570_000, "expand_kernel": 13_050_000,
                           "shrink_kernel": 10_580_000}  # profiles/config2_decode_hbm_traffic_pmc.txt
 
 
