@@ -152,11 +152,21 @@ def cpu_baseline(torch, w, budget_s=15.0):
 COLD_BYTES = 1 << 30   # four times the 256 MB last-level cache of the MI355X
 
 
+def pool_copies(p, n_max):
+    """Copies of a pool's two weight buffers to rotate over, COLD_BYTES in all (at most `n_max` of each): the first is
+    the pool's own."""
+    per = (p.key_buffer.numel() + p.value_buffer.numel()) * p.key_buffer.element_size()
+    n = max(1, min(n_max, -(-COLD_BYTES // per)))
+    return ([p.key_buffer] + [p.key_buffer.clone() for _ in range(n - 1)],
+            [p.value_buffer] + [p.value_buffer.clone() for _ in range(n - 1)])
+
+
 def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0, only_target=None):
     """Per-target timing of the other benchmark configurations and of the headline's decode batch on all seven
     projections of a layer (report only; the JSON line of the default run is config 2's q).  Each target's shrink+expand is replayed back to back on 4 copies of y
     so that the read-modify-write does not hit the same lines (`us`: x and the pool may sit in the
-    last-level cache), and once more over 1 GiB of x / y copies (`us_cold`)."""
+    last-level cache), and once more over 1 GiB of x / y copies and as much of pool copies (`us_cold`: what a
+    forward pass sees, where every layer has its own adapter weights)."""
     report = {}
     for n in ((only,) if only else (1, 2, 3, 4, 5)):
         # 2: the headline's decode batch with LoRA on all seven projections of a layer (the headline itself is its q)
@@ -193,14 +203,15 @@ def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0, only_tar
             n_cold = max(4, -(-COLD_BYTES // (x.numel() * 2 + ycopies[0].numel() * 2)))
             xc = [x.clone() for _ in range(n_cold)]
             yc = [wd.y0[t.name].clone() for _ in range(n_cold)]
+            kc, vc = pool_copies(p, n_cold)
 
             def fc():
-                for xx, yy in zip(xc, yc):
-                    plan.apply(yy, xx, p.key_buffer, p.value_buffer, p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
+                for i, (xx, yy) in enumerate(zip(xc, yc)):
+                    plan.apply(yy, xx, kc[i % len(kc)], vc[i % len(vc)], p.a_start, p.a_len, p.a_loc, t.slot, p.a_scaling)
 
             ms_c, _ = time_graph(torch, fc, 10, 2, use_graph)
             us_cold = ms_c * 1e3 / n_cold
-            del xc, yc
+            del xc, yc, kc, vc
             b, f = w.algorithmic_bytes(t.name), w.flops(t.name)
             rows[t.name] = {"us": round(us, 2), "us_cold": round(us_cold, 2),
                             "shrink_us": round(ms_s * 250, 2), "expand_us": round(ms_e * 250, 2),
@@ -226,10 +237,24 @@ def bench_all_configs(torch, W, LoraPlan, dev, path, use_graph, only=0, only_tar
 
             ms, _ = time_graph(torch, fm, 30, 3, use_graph)
             us = ms * 1e3 / 4
+            n_cold = max(4, -(-COLD_BYTES // (x.numel() * 2 + sum(y.numel() for y in ycopies[0]) * 2)))
+            xc = [x.clone() for _ in range(n_cold)]
+            yc = [[wd.y0[t.name].clone() for t in ts] for _ in range(n_cold)]
+            kc, vc = pool_copies(p, n_cold)
+
+            def fmc():
+                for i, (xx, ys) in enumerate(zip(xc, yc)):
+                    plan.apply_multi(ys, xx, kc[i % len(kc)], vc[i % len(vc)], p.a_start, p.a_len, p.a_loc, slots,
+                                     p.a_scaling)
+
+            ms_c, _ = time_graph(torch, fmc, 10, 2, use_graph)
+            us_cold = ms_c * 1e3 / n_cold
+            del xc, yc, kc, vc
             separate = sum(rows[t.name]["us"] for t in ts)
             # x is read once for the whole group
             b = sum(w.algorithmic_bytes(t.name) for t in ts) - (len(ts) - 1) * w.T * ts[0].h_in * 2
-            groups["+".join(t.name for t in ts)] = {"us": round(us, 2), "separate_us": round(separate, 2),
+            groups["+".join(t.name for t in ts)] = {"us": round(us, 2), "us_cold": round(us_cold, 2),
+                                                    "separate_us": round(separate, 2),
                                                     "bytes": b, "gbps": round(b / us / 1e3, 1),
                                                     "hbm_frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 4)}
             fused_total += us - separate
