@@ -82,6 +82,60 @@ def test_random_shape(dev, seed):
             assert torch.equal(got.cpu(), one), what + " (two targets in one call)"
 
 
+@pytest.mark.parametrize("seed", range(400, 448))
+def test_random_shape_one_launch(dev, seed):
+    """The one-launch op on shapes nobody picked: one to three targets, ranks up to 64, any split-K count, ids with
+    holes, twice on one plan (the hand-off's launch tags move on).  Compared with the oracle, and bit for bit with the
+    two launches of the same split (the library caps K chunks x targets at 16 shrink items per tile, so the
+    two-launch plan is cut with the capped count)."""
+    rnd = random.Random(seed)
+    dtype = rnd.choice([torch.float16, torch.bfloat16])
+    T = rnd.choice([1, 2, 15, 16, 17, 31, 33, 63, 65, 127, 129, 200, 257, 511, 700, 1500])
+    h_in, h_out = rnd.choice(WIDTHS + [5120]), rnd.choice(WIDTHS + [5120])
+    A = rnd.choice([1, 2, 3, 5, 9, 17, 40])
+    ranks = [rnd.choice([8, 16, 24, 32, 40, 48, 64]) for _ in range(A)]
+    n_slots = rnd.choice([1, 2, 4, 4, 5])
+    ks = rnd.choice([2, 3, 4, 5, 8])
+    style = rnd.choice(["random", "sorted", "holes", "one", "none", "zipf"])
+    nt = rnd.choice([1, 1, 2, 3]) if n_slots >= 3 else (rnd.choice([1, 2]) if n_slots == 2 else 1)
+    what = f"seed {seed}: T={T} h_in={h_in} h_out={h_out} ranks={ranks} slots={n_slots} ks={ks} targets={nt} {style} {dtype}"
+    print(what, flush=True)
+    g = torch.Generator().manual_seed(5000 + seed)
+    pool = W.make_pool(ranks, h_in, h_out, dtype, g, True, n_slots=n_slots, std=0.05,
+                       scalings=[0.25 + 0.5 * ((7 * i) % 5) for i in range(A)], heads=1, extra_rows=3)
+    ids = {"random": lambda: torch.randint(0, A, (T,), generator=g),
+           "sorted": lambda: torch.randint(0, A, (T,), generator=g).sort().values,
+           "holes": lambda: torch.randint(-1, A, (T,), generator=g),
+           "one": lambda: torch.full((T,), A - 1, dtype=torch.long),
+           "zipf": lambda: W.zipf_ids(A, T, 0.8, g),
+           "none": lambda: torch.full((T,), -1, dtype=torch.long)}[style]()
+    x = torch.randn(T, h_in, generator=g).to(dtype)
+    slots = rnd.sample(range(n_slots), nt)
+    y0 = [torch.randn(T, h_out, generator=g).to(dtype) for _ in slots]
+    R = max(ranks)
+    pd = pool.to(dev)
+    idx = (pd.a_start, pd.a_len, pd.a_loc)
+    xd, idd = x.to(dev), ids.to(dev)
+    one = LoraPlan(idd, pd.a_start, pd.a_len, R, n_slots=n_slots, hidden=h_in, one_launch=True, ksplit=ks)
+    two = LoraPlan(idd, pd.a_start, pd.a_len, R, n_slots=n_slots, hidden=h_in, one_launch=False, bm_shrink=16,
+                   bm_expand=16, ksplit=min(ks, 16 // nt), reduce_in_expand=True)
+    want = [O.lora_op(y0[i], x, pool.key_buffer, pool.value_buffer, pool.a_start, pool.a_len, pool.a_loc, ids, slot,
+                      pool.a_scaling, n_slots=n_slots) for i, slot in enumerate(slots)]
+    for rep in range(2):
+        y1, y2 = [y.to(dev) for y in y0], [y.to(dev) for y in y0]
+        if nt == 1:
+            one.apply(y1[0], xd, pd.key_buffer, pd.value_buffer, *idx, slots[0], pd.a_scaling)
+            two.apply(y2[0], xd, pd.key_buffer, pd.value_buffer, *idx, slots[0], pd.a_scaling)
+        else:
+            one.apply_multi(y1, xd, pd.key_buffer, pd.value_buffer, *idx, slots, pd.a_scaling)
+            two.apply_multi(y2, xd, pd.key_buffer, pd.value_buffer, *idx, slots, pd.a_scaling)
+        for i in range(nt):
+            got = y1[i].cpu()
+            assert_parity(got, want[i], what + f" target {i} call {rep}")
+            assert torch.equal(got, y2[i].cpu()), what + " (one launch against two)"
+            assert torch.equal(got[ids < 0], y0[i][ids < 0]), what
+
+
 @pytest.mark.parametrize("seed", range(100, 124))
 def test_random_shape_drop_in_bgmv(dev, seed):
     """The same draw through the reference's operator signature (two dispatch_bgmv calls with the
